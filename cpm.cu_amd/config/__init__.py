@@ -2,3 +2,4 @@ from .base import ConfigError, ModelConfig, architecture_name, field_from, read_
 from .minicpm import MiniCPMConfig, RopeScaling, SparseConfig
 from .duvulix import DuvulixConfig
 from .gumodra import GumodraConfig
+from .sagedra import SagedraConfig

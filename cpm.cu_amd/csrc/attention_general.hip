@@ -96,12 +96,15 @@ extern "C" const char* cpmcu_rotate_copy(const void* src, int src_dtype, long ld
 
 #define AG_MAX_HD 1024
 
+// v_share (both attention kernels): runs of v_share neighbouring key heads read one value head (the value pages
+// hold nkv / v_share heads): several score maps over the same values.  1: every key head has its value head.
+
 template <typename T>
 __global__ __launch_bounds__(64) void attention_general_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ kpool, const T* __restrict__ vpool,
     PagedView pv, const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk,
     int hdv, int pool_hdk, int pool_hdv, float scale, int chunk, int window, int keep_first,
-    const float* __restrict__ sink) {
+    const float* __restrict__ sink, int v_share) {
     __shared__ float qs[AG_MAX_HD];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int g = h / (nh / nkv);
@@ -141,7 +144,7 @@ __global__ __launch_bounds__(64) void attention_general_kernel(
         for (int jj = 0; jj < cnt; ++jj) {
             const float pj = __shfl(p, jj, 64);
             const int rj = __shfl(row, jj, 64);
-            const T* vr = vpool + value_index(rj, g, nkv, pool_hdv);
+            const T* vr = vpool + value_index(rj, g / v_share, nkv / v_share, pool_hdv);
 #pragma unroll
             for (int i = 0; i < AG_MAX_HD / 64; ++i) {
                 const int d = lane + 64 * i;
@@ -164,7 +167,9 @@ extern "C" const char* cpmcu_attention_general(const void* q, void* out, int dty
                                                int keep_first, const float* sink, const void* kpool,
                                                const void* vpool,
                                                const int* page_table, int table_width, int page_size,
-                                               const int* positions, const int* tok_slot, hipStream_t stream) {
+                                               const int* positions, const int* tok_slot, int v_share,
+                                               hipStream_t stream) {
+    CPMCU_REQUIRE(v_share >= 1 && nkv % v_share == 0, "attention_general: %d key heads do not share values in runs of %d", nkv, v_share);
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && hdk > 0 && hdv > 0,
                   "attention_general: empty shape n=%d heads=%d kv_heads=%d key size=%d value size=%d", n, nh, nkv, hdk, hdv);
     CPMCU_REQUIRE(nh % nkv == 0, "attention_general: %d heads are not a multiple of %d kv heads", nh, nkv);
@@ -183,12 +188,12 @@ extern "C" const char* cpmcu_attention_general(const void* q, void* out, int dty
         attention_general_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, (float*)out, (const float*)kpool,
                                                                  (const float*)vpool, pv, positions, tok_slot, nh, nkv,
                                                                  hdk, hdv, pool_hdk, pool_hdv, scale, chunk, window,
-                                                                 keep_first, sink);
+                                                                 keep_first, sink, v_share);
     else if (dtype == CPMCU_BF16)
         attention_general_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kpool,
                                                                   (const bf16_t*)vpool, pv, positions, tok_slot, nh,
                                                                   nkv, hdk, hdv, pool_hdk, pool_hdv, scale, chunk, window,
-                                                                  keep_first, sink);
+                                                                  keep_first, sink, v_share);
     else
         CPMCU_FAIL("attention_general: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("attention_general");
@@ -225,7 +230,7 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk, int hdv,
     int pool_hdk, int pool_hdv, float scale_log2e, int chunk, int window, int keep_first, const float* __restrict__ sink,
-    int n_splits, int n_tokens, const int* __restrict__ tiles, int n_tiles, int tpt, int rpt) {
+    int n_splits, int n_tokens, const int* __restrict__ tiles, int n_tiles, int tpt, int rpt, int v_share) {
     extern __shared__ __align__(16) unsigned char smem[];
     static_assert(NW == 1 || TW == 1, "either the wavefronts of a workgroup share a token or each has its own");
     const int ksteps = (pool_hdk + 31) >> 5, dtn = pool_hdv >> 4;
@@ -286,7 +291,7 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
         const int key0 = (c < ckeep ? c : cfirst + (c - ckeep)) << 5;
         const long pchunk = paged_row(pv, slot, key0) >> 5;
         const bf16_t* kp = kpool + (pchunk * nkv + kvh) * kchunk + lane_off;
-        const bf16_t* vp = vtpool + (pchunk * nkv + kvh) * vchunk + lane_off;
+        const bf16_t* vp = vtpool + (pchunk * (nkv / v_share) + kvh / v_share) * vchunk + lane_off;
         // the values are asked for first: they arrive behind the scores' work.  No load stands in a branch
         // (lanes beyond the head's features read its first ones and are zeroed by a select), so that the
         // compiler keeps several steps' loads in flight.
@@ -474,8 +479,9 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
                                                     const float* sink, const void* kpool, const void* vtpool,
                                                     const int* page_table, int table_width, int page_size,
                                                     const int* positions, const int* tok_slot, int n_splits,
-                                                    const int* tiles, int n_tiles, int tokens_per_tile,
+                                                    const int* tiles, int n_tiles, int tokens_per_tile, int v_share,
                                                     hipStream_t stream) {
+    CPMCU_REQUIRE(v_share >= 1 && nkv % v_share == 0, "attention_general_mfma: %d key heads do not share values in runs of %d", nkv, v_share);
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_general_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
     CPMCU_REQUIRE(hdk > 0 && hdk % 8 == 0 && hdk <= 1024 && hdv > 0 && hdv <= 512,
                   "attention_general_mfma: key size %d (a multiple of 8 up to 1024) / value size %d (up to 512) have no "
@@ -516,7 +522,7 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
     attention_general_mfma_kernel<DTMv, NWv, TWv, VSv><<<grid, NWv * TWv * 64, lds, stream>>>(                   \
         (const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
         positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, window, keep_first, sink, n_splits, n,    \
-        tiles, n_tiles, tpt, rpt)
+        tiles, n_tiles, tpt, rpt, v_share)
     if (vs) {
         if (dtm == 4) LAUNCH(4, 4, 1, true);
         else LAUNCH(8, 4, 1, true);
@@ -628,14 +634,16 @@ extern "C" const char* cpmcu_qkv_rotate_store(const void* qkv, long ld, int dtyp
 //   * q heads and k heads are divided by their root mean square (eps inside the root) and multiplied by a weight
 //     of dk numbers shared by the heads (q_norm_w, k_norm_w; either may be absent), before the rotation;
 //   * with values_from_keys the row holds no v: the value pages receive k as projected (with its bias, before norm
-//     and rotation), so dv == dk.
+//     and rotation), so dv == dk;
+//   * with norm_after q and k heads are rotated first and then divided by their root mean square (times the
+//     weight, if one is given).
 template <typename T>
 __global__ __launch_bounds__(64) void qkv_norm_rotate_store_kernel(
     const T* __restrict__ qkv, long ld, const float* __restrict__ bias, T* __restrict__ q_out, int nh, int nkv, int dk,
     int dv, int rot_dims, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
     int values_from_keys, const int* __restrict__ positions, const int* __restrict__ tok_slot,
     const float* __restrict__ inv_freq, float mag, T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv,
-    int pool_hdk, int pool_hdv) {
+    int pool_hdk, int pool_hdv, int norm_after) {
     __shared__ float hs[AG_MAX_HD];
     const long t = blockIdx.x;
     const int y = blockIdx.y, lane = threadIdx.x;
@@ -662,7 +670,24 @@ __global__ __launch_bounds__(64) void qkv_norm_rotate_store_kernel(
         for (int i = lane; i < width; i += 64) vd[value_d_offset(i)] = from_f32<T>(hs[i]);
     }
     const float* nw = is_q ? q_norm_w : k_norm_w;
-    if (nw) {
+    if (norm_after) {
+        // the rotation first (in place, in float), then the division by the rotated head's root mean square
+        __syncthreads();
+        const int half = rot_dims / 2;
+        for (int i = lane; i < half; i += 64) {
+            const float ang = (float)pos * inv_freq[i];
+            const float cs = cosf(ang) * mag, sn = sinf(ang) * mag;
+            const float u = hs[i], v = hs[i + half];
+            hs[i] = u * cs - v * sn;
+            hs[i + half] = v * cs + u * sn;
+        }
+        __syncthreads();
+        float s2 = 0.f;
+        for (int i = lane; i < width; i += 64) s2 += hs[i] * hs[i];
+        const float r = 1.0f / sqrtf(wave_sum(s2) / (float)width + eps);
+        for (int i = lane; i < width; i += 64) hs[i] = hs[i] * r * (nw ? nw[i] : 1.0f);
+        rot_dims = 0;
+    } else if (nw) {
         const float r = 1.0f / sqrtf(wave_sum(ss) / (float)width + eps);
         for (int i = lane; i < width; i += 64) hs[i] = hs[i] * r * nw[i];
     }
@@ -677,7 +702,7 @@ extern "C" const char* cpmcu_qkv_norm_rotate_store(const void* qkv, long ld, int
                                                    int values_from_keys, const int* positions, const int* tok_slot,
                                                    const float* inv_freq, float mag, void* kpool, void* vpool,
                                                    const int* page_table, int table_width, int page_size, int pool_hdk,
-                                                   int pool_hdv, int write_kv, hipStream_t stream) {
+                                                   int pool_hdv, int write_kv, int norm_after, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "qkv_norm_rotate_store: empty shape");
     CPMCU_REQUIRE(dk <= AG_MAX_HD && dv <= AG_MAX_HD, "qkv_norm_rotate_store: key size %d / value size %d (up to %d are taken)",
                   dk, dv, AG_MAX_HD);
@@ -696,11 +721,12 @@ extern "C" const char* cpmcu_qkv_norm_rotate_store(const void* qkv, long ld, int
     if (dtype == CPMCU_F32)
         qkv_norm_rotate_store_kernel<float><<<grid, 64, 0, stream>>>(
             (const float*)qkv, ld, bias, (float*)q_out, nh, nkv, dk, dv, rot_dims, q_norm_w, k_norm_w, eps, values_from_keys,
-            positions, tok_slot, inv_freq, mag, (float*)kpool, (float*)vpool, pv, pool_hdk, pool_hdv);
+            positions, tok_slot, inv_freq, mag, (float*)kpool, (float*)vpool, pv, pool_hdk, pool_hdv, norm_after);
     else if (dtype == CPMCU_BF16)
         qkv_norm_rotate_store_kernel<bf16_t><<<grid, 64, 0, stream>>>(
             (const bf16_t*)qkv, ld, bias, (bf16_t*)q_out, nh, nkv, dk, dv, rot_dims, q_norm_w, k_norm_w, eps,
-            values_from_keys, positions, tok_slot, inv_freq, mag, (bf16_t*)kpool, (bf16_t*)vpool, pv, pool_hdk, pool_hdv);
+            values_from_keys, positions, tok_slot, inv_freq, mag, (bf16_t*)kpool, (bf16_t*)vpool, pv, pool_hdk, pool_hdv,
+            norm_after);
     else
         CPMCU_FAIL("qkv_norm_rotate_store: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("qkv_norm_rotate_store");

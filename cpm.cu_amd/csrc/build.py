@@ -30,11 +30,12 @@ MODULES: Dict[str, List[str]] = {
     "attention": ["attention.hip"],
     "sparse": ["sparse.hip"],
     "qkv": ["qkv_rope.hip", "strip.hip"],
-    "norms": ["norms.hip", "residual.hip"],
+    "norms": ["norms.hip", "residual.hip", "streams.hip"],
     "ssm": ["ssm.hip"],
     "mlstm": ["mlstm.hip"],
+    "delta": ["delta.hip"],
     "moe": ["moe.hip"],
-    "attention_general": ["attention_general.hip"],
+    "attention_general": ["attention_general.hip", "diff_attention.hip"],
 }
 HEADERS = ["common.h"]
 # headers of single libraries

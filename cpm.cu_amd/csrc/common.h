@@ -43,6 +43,14 @@ template <typename T> __host__ __device__ inline T from_f32(float f);
 template <> __host__ __device__ inline float from_f32<float>(float f) { return f; }
 template <> __host__ __device__ inline bf16_t from_f32<bf16_t>(float f) { return f32_to_bf16(f); }
 
+// Nonlinearity of a gated feed-forward's gate, act(g) * up.  Both kinds are g * sigmoid(s(g)): SiLU with s(g) = g,
+// the tanh form of GELU with s(g) = 2 sqrt(2/pi) (g + 0.044715 g^3), since 0.5 (1 + tanh z) = sigmoid(2 z).
+enum { CPMCU_ACT_SILU = 0, CPMCU_ACT_GELU_TANH = 1 };
+__host__ __device__ inline float gate_arg(float g, int act) {
+    return act == CPMCU_ACT_GELU_TANH ? 1.5957691216057308f * (g + 0.044715f * g * g * g) : g;
+}
+__device__ inline float gate_act(float g, int act) { return g / (1.0f + expf(-gate_arg(g, act))); }
+
 // Max / sum over the four rows of 16 lanes of a wavefront (lanes that differ in bits 4 and 5 only); every
 // lane gets the result.  gfx950's row swaps exchange rows between two registers inside the vector unit:
 // swapping a value with itself leaves (row 0, row 0, row 2, row 2) and (row 1, row 1, row 3, row 3).

@@ -33,6 +33,21 @@ extern "C" const char* cpmcu_embed(const void* table, int dtype, const int* ids,
     return nullptr;
 }
 
+// logits <- cap * tanh(logits / cap), in place (a soft cap on the head's output)
+__global__ void softcap_kernel(float* __restrict__ x, long total, float cap) {
+    const float inv = 1.0f / cap;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x)
+        x[i] = cap * tanhf(x[i] * inv);
+}
+
+extern "C" const char* cpmcu_softcap(float* x, long total, float cap, hipStream_t stream) {
+    CPMCU_REQUIRE(total > 0 && x && cap > 0.f, "softcap: empty shape or a cap that is not positive");
+    const long wgs = (total + 255) / 256;
+    softcap_kernel<<<(unsigned)(wgs < 65535L * 16 ? wgs : 65535L * 16), 256, 0, stream>>>(x, total, cap);
+    CPMCU_LAUNCH_CHECK("softcap");
+    return nullptr;
+}
+
 // ---------------------------------------------------------------------------
 // x += bscale * sum_p branch[p]   (written back unless `rows` selects rows)
 // out = x * rsqrt(mean(x^2) + eps) * w
@@ -300,18 +315,18 @@ extern "C" const char* cpmcu_add_norm_columns(float* x, const void* branch, int 
 }
 
 // ---------------------------------------------------------------------------
-// out[r,c] = silu(gu[r,c]) * gu[r,c+I],  silu(g) = g / (1 + exp(-g))
+// out[r,c] = act(gu[r,c]) * gu[r,c+I],  act = SiLU, silu(g) = g / (1 + exp(-g)), or the tanh form of GELU
 // (reference: src/model/activation.cuh:6-18, gate columns first, then up)
 // ---------------------------------------------------------------------------
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, long n, int I) {
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, long n, int I, int act) {
     const long total = n * I;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
         const long r = i / I;
         const int c = (int)(i - r * I);
         const float g = to_f32(gu[r * 2 * I + c]);
         const float u = to_f32(gu[r * 2 * I + I + c]);
-        out[i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+        out[i] = from_f32<T>(gate_act(g, act) * u);
     }
 }
 
@@ -321,7 +336,7 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, l
 // (2^-22 relative; the 32-bit engine's kernel above keeps expf and a true division).
 template <int U>
 __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
-                                                              long n, int I) {
+                                                              long n, int I, int act) {
     const int I8 = I / 8;
     const long total = n * I8;
     const long base = (long)blockIdx.x * (256 * U) + threadIdx.x;
@@ -345,8 +360,8 @@ __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __re
         for (int j = 0; j < 4; ++j) {
             const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
             const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
-            const float s0 = g0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g0));
-            const float s1 = g1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g1));
+            const float s0 = g0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * gate_arg(g0, act)));
+            const float s1 = g1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * gate_arg(g1, act)));
             const bf16_t a = f32_to_bf16(s0 * u0);
             const bf16_t b = f32_to_bf16(s1 * u1);
             ow[j] = (uint32_t)a.v | ((uint32_t)b.v << 16);
@@ -355,19 +370,20 @@ __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __re
     }
 }
 
-extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int n, int I, hipStream_t stream) {
+extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int n, int I, int act, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && I > 0, "silu_mul: empty shape n=%d I=%d", n, I);
+    CPMCU_REQUIRE(act == CPMCU_ACT_SILU || act == CPMCU_ACT_GELU_TANH, "silu_mul: unknown nonlinearity %d", act);
     if (dtype == CPMCU_BF16 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
         const long total8 = (long)n * (I / 8);
         // many rows: 4 pieces a thread in flight; few: one, for more workgroups
         if (total8 >= 4L * 256 * 2048) {
             const long wgs = (total8 + 4 * 256 - 1) / (4 * 256);
             CPMCU_REQUIRE(wgs <= 0x7fffffffL, "silu_mul: %d rows of %d columns exceed the launch grid", n, I);
-            silu_mul_bf16x8_kernel<4><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I);
+            silu_mul_bf16x8_kernel<4><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I, act);
         } else {
             const long wgs = (total8 + 255) / 256;
             CPMCU_REQUIRE(wgs <= 0x7fffffffL, "silu_mul: %d rows of %d columns exceed the launch grid", n, I);
-            silu_mul_bf16x8_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I);
+            silu_mul_bf16x8_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I, act);
         }
         CPMCU_LAUNCH_CHECK("silu_mul");
         return nullptr;
@@ -376,9 +392,9 @@ extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int 
     const int block = 256;
     const int grid = (int)((total + block - 1) / block < 65535 * 16 ? (total + block - 1) / block : 65535 * 16);
     if (dtype == CPMCU_F32)
-        silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, n, I);
+        silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, n, I, act);
     else if (dtype == CPMCU_BF16)
-        silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I);
+        silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I, act);
     else
         CPMCU_FAIL("silu_mul: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("silu_mul");

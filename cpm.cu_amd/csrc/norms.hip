@@ -24,6 +24,7 @@ __device__ inline float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
 // grid (rows, groups); out[r, g*W + c] = v * rsqrt(mean_g(v^2) + eps) * weight[g*W + c], v = x * silu(z) if z and
 // gate_after == 0; with gate_after the statistics are those of x alone and the result is multiplied by sigmoid(z)
+// (gate_after == 1) or by silu(z) (gate_after == 2)
 template <typename XT, typename ZT, typename OT>
 __global__ __launch_bounds__(256) void rms_norm_groups_kernel(const XT* __restrict__ x, long ldx,
                                                               const ZT* __restrict__ z, long ldz,
@@ -52,7 +53,7 @@ __global__ __launch_bounds__(256) void rms_norm_groups_kernel(const XT* __restri
         if (before) v *= silu_f(to_f32(zr[c]));
         v *= rs;
         if (weight) v *= weight[(long)g * W + c];
-        if (zr && gate_after) v *= 1.0f / (1.0f + expf(-to_f32(zr[c])));
+        if (zr && gate_after) v *= gate_after == 2 ? silu_f(to_f32(zr[c])) : 1.0f / (1.0f + expf(-to_f32(zr[c])));
         orow[c] = from_f32<OT>(v);
     }
 }

@@ -81,3 +81,31 @@ extern "C" const char* cpmcu_bias_sum(const void* a, int dtype, int parts, long 
     CPMCU_LAUNCH_CHECK("bias_sum");
     return nullptr;
 }
+
+// out = a * sigmoid(g), element by element: an attention's heads side by side times a gate that is a projection
+// of the mixer's input (g may be columns of a wider projection); the sigmoid in float.
+template <typename T>
+__global__ __launch_bounds__(256) void sigmoid_gate_kernel(const T* __restrict__ a, const T* __restrict__ g, long ldg,
+                                                           T* __restrict__ out, long total, int W) {
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+        const long t = i / W;
+        const int c = (int)(i - t * W);
+        out[i] = from_f32<T>(to_f32(a[i]) / (1.0f + expf(-to_f32(g[t * ldg + c]))));
+    }
+}
+
+extern "C" const char* cpmcu_sigmoid_gate(const void* a, const void* g, long ldg, void* out, int dtype, int n, int W,
+                                          hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && W > 0 && a && g && out && ldg >= W, "sigmoid_gate: empty shape or rows too short");
+    const long total = (long)n * W;
+    const long wgs = (total + 255) / 256;
+    const unsigned grid = (unsigned)(wgs < 65535L * 16 ? wgs : 65535L * 16);
+    if (dtype == CPMCU_F32)
+        sigmoid_gate_kernel<float><<<grid, 256, 0, stream>>>((const float*)a, (const float*)g, ldg, (float*)out, total, W);
+    else if (dtype == CPMCU_BF16)
+        sigmoid_gate_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)g, ldg, (bf16_t*)out, total, W);
+    else
+        CPMCU_FAIL("sigmoid_gate: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("sigmoid_gate");
+    return nullptr;
+}

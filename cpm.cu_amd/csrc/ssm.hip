@@ -1,8 +1,10 @@
 // State-space (Mamba-2 style) sequence mixing over a packed batch, with per-slot state:
 //
 //  * conv_silu_kernel: causal convolution per channel over a sequence's tokens (taps weights a channel, the last
-//    column is the current token's; inputs before the sequence's start are zero) followed by SiLU.  The
-//    sequence's last taps-1 inputs live in the slot's state, so a step continues where the last one ended.
+//    column is the current token's; inputs before the sequence's start are zero) followed by SiLU, or by nothing.
+//    The sequence's last taps-1 inputs live in the slot's state, so a step continues where the last one ended.
+//    With in_bias the convolution's inputs are u + in_bias (a projection's bias that is still to be added); the
+//    state holds them with it, and the inputs before the start stay zero.
 //  * conv_state_kernel: moves the step's last inputs into that state (after the convolution has read it); for
 //    steps of at most 16 tokens a sequence the convolution's kernel does that itself.
 //  * ssm_scan_kernel: the recurrence, per head h (group g = h / (heads / groups)):
@@ -25,7 +27,8 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u
                                                         const float* __restrict__ bias,
                                                         const float* state, float* __restrict__ out,
                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_slot,
-                                                        int C, int taps, float* state_out) {
+                                                        int C, int taps, float* state_out,
+                                                        const float* __restrict__ in_bias, int plain) {
     const int b = blockIdx.x;
     const int start = cu_q[b], q = cu_q[b + 1] - start;
     const int slot = seq_slot[b];
@@ -34,14 +37,15 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u
     const int i0 = blockIdx.y * 16, i1 = min(i0 + 16, q);
     const float* st = state + (long)slot * (taps - 1) * C + c;        // [slot][taps-1][C]
     const float bs = bias ? bias[c] : 0.f;
+    const float ib = in_bias ? in_bias[c] : 0.f;
     for (int i = i0; i < i1; ++i) {
         float acc = bs;
         for (int k = 0; k < taps; ++k) {
             const int j = i - (taps - 1 - k);                          // local index of the input this tap reads
-            const float in = j >= 0 ? to_f32(u[(long)(start + j) * ldu + c]) : st[(long)(taps - 1 + j) * C];
+            const float in = j >= 0 ? to_f32(u[(long)(start + j) * ldu + c]) + ib : st[(long)(taps - 1 + j) * C];
             acc += weight[(long)c * taps + k] * in;
         }
-        out[(long)(start + i) * C + c] = silu_f(acc);
+        out[(long)(start + i) * C + c] = plain ? acc : silu_f(acc);
     }
     // steps of at most 16 tokens a sequence (decode steps): this thread alone has read its channel's state, so
     // it moves the step's last inputs into it itself and the second kernel is not launched
@@ -49,7 +53,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u
         float* so = state_out + (long)slot * (taps - 1) * C + c;
         for (int j = 0; j < taps - 1; ++j) {
             const int i = q - (taps - 1) + j;
-            so[(long)j * C] = i >= 0 ? to_f32(u[(long)(start + i) * ldu + c]) : so[(long)(j + q) * C];
+            so[(long)j * C] = i >= 0 ? to_f32(u[(long)(start + i) * ldu + c]) + ib : so[(long)(j + q) * C];
         }
     }
 }
@@ -60,22 +64,24 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u
 template <typename UT>
 __global__ __launch_bounds__(256) void conv_state_kernel(const UT* __restrict__ u, long ldu, float* __restrict__ state,
                                                          const int* __restrict__ cu_q, const int* __restrict__ seq_slot,
-                                                         int C, int taps) {
+                                                         int C, int taps, const float* __restrict__ in_bias) {
     const int b = blockIdx.x;
     const int start = cu_q[b], q = cu_q[b + 1] - start;
     const int slot = seq_slot[b];
     const int c = blockIdx.y * blockDim.x + threadIdx.x;
     if (c >= C) return;
     float* st = state + (long)slot * (taps - 1) * C + c;
+    const float ib = in_bias ? in_bias[c] : 0.f;
     for (int j = 0; j < taps - 1; ++j) {
         const int i = q - (taps - 1) + j;
-        st[(long)j * C] = i >= 0 ? to_f32(u[(long)(start + i) * ldu + c]) : st[(long)(j + q) * C];
+        st[(long)j * C] = i >= 0 ? to_f32(u[(long)(start + i) * ldu + c]) + ib : st[(long)(j + q) * C];
     }
 }
 
 extern "C" const char* cpmcu_conv_silu(const void* u, long ldu, int u_dtype, const float* weight, const float* bias,
                                        float* state, float* out, const int* cu_q, const int* seq_slot, int n_seqs,
-                                       int max_q, int C, int taps, int update_state, hipStream_t stream) {
+                                       int max_q, int C, int taps, int update_state, const float* in_bias, int plain,
+                                       hipStream_t stream) {
     CPMCU_REQUIRE(n_seqs > 0 && max_q > 0 && C > 0 && taps >= 1, "conv_silu: empty shape sequences=%d tokens=%d channels=%d taps=%d",
                   n_seqs, max_q, C, taps);
     CPMCU_REQUIRE(ldu >= C, "conv_silu: rows of %ld elements cannot hold %d channels", ldu, C);
@@ -87,13 +93,13 @@ extern "C" const char* cpmcu_conv_silu(const void* u, long ldu, int u_dtype, con
     const bool moves = update_state && taps > 1;
     float* fused = (moves && tb == 1) ? state : nullptr;
     if (u_dtype == CPMCU_F32) {
-        conv_silu_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps, fused);
+        conv_silu_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps, fused, in_bias, plain);
         if (moves && !fused)
-            conv_state_kernel<float><<<grid2, 256, 0, stream>>>((const float*)u, ldu, state, cu_q, seq_slot, C, taps);
+            conv_state_kernel<float><<<grid2, 256, 0, stream>>>((const float*)u, ldu, state, cu_q, seq_slot, C, taps, in_bias);
     } else if (u_dtype == CPMCU_BF16) {
-        conv_silu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps, fused);
+        conv_silu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps, fused, in_bias, plain);
         if (moves && !fused)
-            conv_state_kernel<bf16_t><<<grid2, 256, 0, stream>>>((const bf16_t*)u, ldu, state, cu_q, seq_slot, C, taps);
+            conv_state_kernel<bf16_t><<<grid2, 256, 0, stream>>>((const bf16_t*)u, ldu, state, cu_q, seq_slot, C, taps, in_bias);
     } else {
         CPMCU_FAIL("conv_silu: unknown dtype %d", u_dtype);
     }

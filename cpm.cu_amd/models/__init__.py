@@ -3,3 +3,4 @@ from .decoder import DecoderModel, Run, sequential_schedule
 from . import minicpm
 from . import duvulix
 from . import gumodra
+from . import sagedra

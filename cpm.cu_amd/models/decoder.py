@@ -17,6 +17,7 @@ from typing import List, Optional, Sequence
 
 import torch
 
+from .. import ops
 from ..cache.paged import CacheNeeds
 from ..parts.base import Block, Norm, Part, ResidualStream, Runtime, StepContext, branch_for
 from ..parts.embedding import LMHead, TokenEmbedding
@@ -35,8 +36,11 @@ def sequential_schedule(n_layers: int) -> List[Run]:
 
 class DecoderModel(Part):
     def __init__(self, config, embedding: TokenEmbedding, layers: Sequence[Block], final_norm: Norm, head: LMHead,
-                 schedule: Optional[Sequence[Run]] = None):
+                 schedule: Optional[Sequence[Run]] = None, streams: Optional[int] = None):
+        """``streams``: the residual is that many rows a token (hyper-connections), all equal to the embedding's
+        output at the start; the blocks mix them, and the last norm reads their sum."""
         self.config = config
+        self.streams = int(streams) if streams else None
         self.embedding = embedding
         self.layers = list(layers)
         self.final_norm = final_norm
@@ -77,13 +81,22 @@ class DecoderModel(Part):
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """float32 logits [R, V] at ctx.logit_rows; the step's tokens enter the cache."""
         with ctx.timed("embed"):
-            stream = ResidualStream(self.embedding.forward(ctx))
+            x = self.embedding.forward(ctx)
+            if self.streams:
+                lanes = ctx.ws.get("residual.streams", (self.streams,) + tuple(x.shape), torch.float32)
+                ops.streams_fill(x, lanes)
+                x = lanes
+            stream = ResidualStream(x)
         for r in self.schedule:
             self.layers[r.layer].forward(stream, ctx, ctx.cache.view(r.cache) if ctx.cache is not None else None,
                                          r.writes_cache)
         if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
             return None
         with ctx.timed("head"):
-            y = self.final_norm.forward(stream.x, branch_for(self.final_norm, stream.take_pending()),
-                                        stream.pending_scale, ctx, rows=ctx.logit_rows, tag="final.y")
+            if self.streams:
+                y = self.final_norm.forward_streams(stream.x, stream.take_pending(), None, ctx, rows=ctx.logit_rows,
+                                                    tag="final.y")
+            else:
+                y = self.final_norm.forward(stream.x, branch_for(self.final_norm, stream.take_pending()),
+                                            stream.pending_scale, ctx, rows=ctx.logit_rows, tag="final.y")
             return self.head.forward(y, ctx)

@@ -172,14 +172,26 @@ def add_norm_columns(x: torch.Tensor, branch: Optional[torch.Tensor], branch_sca
                                                  c_int(H), _stream()))
 
 
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor):
-    """out[r,c] = silu(gate_up[r,c]) * gate_up[r,c+I];  gate_up [n,2I], out [n,I]."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def _act(activation: str) -> int:
+    try:
+        return GATE_ACTIVATIONS[activation]
+    except KeyError:
+        raise KernelError(f"gate nonlinearity '{activation}' is not supported ({sorted(GATE_ACTIVATIONS)})") from None
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu"):
+    """out[r,c] = act(gate_up[r,c]) * gate_up[r,c+I];  gate_up [n,2I], out [n,I]; act is SiLU or, with
+    activation 'gelu_tanh', 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))."""
     _need(gate_up, "silu_mul input", shape=(None, None))
     n, two_i = gate_up.shape
     if two_i % 2:
         raise KernelError(f"silu_mul: input width {two_i} is odd")
     _need(out, "silu_mul out", gate_up.dtype, (n, two_i // 2))
-    _check(_fn("core", "cpmcu_silu_mul")(_p(gate_up), _p(out), c_int(_code(out)), c_int(n), c_int(two_i // 2), _stream()))
+    _check(_fn("core", "cpmcu_silu_mul")(_p(gate_up), _p(out), c_int(_code(out)), c_int(n), c_int(two_i // 2),
+                                         c_int(_act(activation)), _stream()))
 
 
 def rope_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, hd: int, positions: torch.Tensor,
@@ -457,11 +469,11 @@ def _ld(t: torch.Tensor, name: str) -> int:
 
 
 def rms_norm_groups(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out: torch.Tensor, groups: int = 1,
-                    gate: Optional[torch.Tensor] = None, gate_after: bool = False,
+                    gate: Optional[torch.Tensor] = None, gate_after=False,
                     divisor: Optional[torch.Tensor] = None):
     """out[r] = v / sqrt(mean(v^2) + eps) * weight, group by group (``groups`` equal parts of a row, each by its
     own root mean square), v = x * silu(gate) when a gate is given (the gate comes before the norm); with
-    ``gate_after`` v = x and the result is multiplied by sigmoid(gate) instead.  ``divisor`` (float32 [n, groups]):
+    ``gate_after`` v = x and the result is multiplied by sigmoid(gate) instead (by silu(gate) with gate_after="silu").  ``divisor`` (float32 [n, groups]):
     a group's values are divided by its number first.  x, gate and out may be column slices of wider tensors;
     statistics in float."""
     ldx, ldo = _ld(x, "norm x"), _ld(out, "norm out")
@@ -482,7 +494,7 @@ def rms_norm_groups(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
     _check(_fn("norms", "cpmcu_rms_norm_groups")(_p(x), c_long(ldx), c_int(_code(x)), _p(gate), c_long(ldz),
                                                  c_int(_code(gate) if gate is not None else 0), _p(weight), _p(out),
                                                  c_long(ldo), c_int(_code(out)), c_int(n), c_int(groups),
-                                                 c_int(width // groups), c_float(eps), c_int(1 if gate_after else 0),
+                                                 c_int(width // groups), c_float(eps), c_int(2 if gate_after == "silu" else (1 if gate_after else 0)),
                                                  _p(divisor), _stream()))
 
 
@@ -533,17 +545,22 @@ def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float, out: torch.Tensor
 
 
 def conv_silu(u: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
-              out: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor, max_q: int, update_state: bool = True):
+              out: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor, max_q: int, update_state: bool = True,
+              in_bias: Optional[torch.Tensor] = None, activation: bool = True):
     """Causal convolution per channel over each sequence's tokens, then SiLU.  u [n,C] (may be a column slice),
     weight float32 [C,taps] (last column = the current token's), state float32 [slots, taps-1, C] = each slot's
     last inputs (zeros before a sequence's start), out float32 [n,C].  cu_q int32 [B+1], seq_slot int32 [B];
-    max_q: the longest run of tokens a sequence brings.  The state moves on to the step's last inputs."""
+    max_q: the longest run of tokens a sequence brings.  The state moves on to the step's last inputs.
+    in_bias (float32 [C]): the inputs are u + in_bias (a projection's bias not yet added; the state holds them
+    with it).  Without ``activation`` the convolution's result is written as it is."""
     ldu = _ld(u, "conv input")
     n, C = u.shape
     _need(weight, "conv weight", torch.float32, (C, None))
     taps = weight.shape[1]
     if bias is not None:
         _need(bias, "conv bias", torch.float32, (C,))
+    if in_bias is not None:
+        _need(in_bias, "conv input bias", torch.float32, (C,))
     if taps > 1:
         _need(state, "conv state", torch.float32, (None, taps - 1, C))
     _need(out, "conv out", torch.float32, (n, C))
@@ -552,7 +569,8 @@ def conv_silu(u: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
     _need(seq_slot, "conv sequence slots", torch.int32, (B,))
     _check(_fn("ssm", "cpmcu_conv_silu")(_p(u), c_long(ldu), c_int(_code(u)), _p(weight), _p(bias), _p(state), _p(out),
                                          _p(cu_q), _p(seq_slot), c_int(B), c_int(max_q), c_int(C), c_int(taps),
-                                         c_int(1 if update_state else 0), _stream()))
+                                         c_int(1 if update_state else 0), _p(in_bias),
+                                         c_int(0 if activation else 1), _stream()))
 
 
 def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A_log: torch.Tensor, D: torch.Tensor,
@@ -655,12 +673,14 @@ def qkv_norm_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: 
                           kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor],
                           page_table: Optional[torch.Tensor], page_size: int, write_kv: bool = True,
                           bias: Optional[torch.Tensor] = None, q_norm: Optional[torch.Tensor] = None,
-                          k_norm: Optional[torch.Tensor] = None, eps: float = 0.0, values_from_keys: bool = False):
+                          k_norm: Optional[torch.Tensor] = None, eps: float = 0.0, values_from_keys: bool = False,
+                          norm_after: bool = False):
     """qkv_rotate_store with what some designs put between projection and rotation: ``bias`` (float32, as wide as
     a row of qkv) is added; q heads and k heads are divided by their root mean square (eps inside the root) and
     multiplied by a weight of dk numbers shared by the heads (q_norm, k_norm, float32 [dk]); with
     values_from_keys a row is [q | k] only and the value pages receive k as projected (with its bias, before norm
-    and rotation)."""
+    and rotation).  With norm_after the q and k heads are rotated first and then divided by their root mean square
+    (times q_norm / k_norm where given, by nothing else where not)."""
     ld = _ld(qkv, "qkv")
     n = qkv.shape[0]
     width = nh * dk + ((nkv * dk + (0 if values_from_keys else nkv * dv)) if write_kv else 0)
@@ -693,7 +713,7 @@ def qkv_norm_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: 
         c_int(rot_dims), _p(q_norm), _p(k_norm), c_float(eps), c_int(1 if values_from_keys else 0), _p(positions),
         _p(tok_slot), _p(inv_freq), c_float(mag), _p(kpool if write_kv else None), _p(vpool if write_kv else None),
         _p(page_table if write_kv else None), c_int(tw), c_int(page_size), c_int(pk), c_int(pv),
-        c_int(1 if write_kv else 0), _stream()))
+        c_int(1 if write_kv else 0), c_int(1 if norm_after else 0), _stream()))
 
 
 def _parts_of(t: torch.Tensor, n: int, H: int, name: str):
@@ -769,6 +789,165 @@ def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: in
                                             c_float(cap), c_float(q_scale), _p(S), _p(n_state), _p(m_state), _p(y),
                                             _p(den), _p(cu_q), _p(seq_slot), c_int(B), c_int(heads), c_int(d), c_int(dv),
                                             c_int(1 if write_state else 0), _stream()))
+
+
+def streams_fill(x: torch.Tensor, streams: torch.Tensor):
+    """streams[s] = x for every s: a residual of several streams starts as copies of the embedding's output.
+    x float32 [n, H], streams float32 [S, n, H]."""
+    _need(x, "streams source", torch.float32, (None, None))
+    n, H = x.shape
+    _need(streams, "residual streams", torch.float32, (None, n, H))
+    _check(_fn("norms", "cpmcu_streams_fill")(_p(x), _p(streams), c_long(n * H), c_int(streams.shape[0]), _stream()))
+
+
+def streams_norm(x: torch.Tensor, branch: Optional[torch.Tensor], branch_bias: Optional[torch.Tensor],
+                 branch_scale: float, mix: Optional[torch.Tensor], out_weights: Optional[torch.Tensor],
+                 read: Optional[torch.Tensor], weight: torch.Tensor, eps: float, out: torch.Tensor,
+                 rows: Optional[torch.Tensor] = None, rms: bool = False):
+    """The residual add and the norm that follows it, for a residual of S >= 1 streams x float32 [S, n, H] (or
+    [n, H], one stream).  With a branch y = branch_scale * branch (+ branch_bias; summed over the leading axis if
+    it is [P, n, H]):  x_t <- sum_s mix[s, t] x_s + out_weights[t] * y  (mix float32 [S, S] indexed [from, to],
+    None: each stream keeps itself; out_weights float32 [S], None: ones), all streams at once, in place.  Then
+    u = sum_t read[t] x_t (read float32 [S], None: the plain sum) and out = layer norm without bias of u,
+    (u - mean) / sqrt(variance + eps) * weight, or with ``rms`` u / sqrt(mean(u^2) + eps) * weight.  With ``rows``
+    (int32 [R]) only those rows are computed, into out [R, H], and x is left as it was."""
+    if x.dim() == 2:
+        _need(x, "residual", torch.float32, (None, None))
+        S, (n, H) = 1, x.shape
+    else:
+        _need(x, "residual streams", torch.float32, (None, None, None))
+        S, n, H = x.shape
+    _need(weight, "norm weight", torch.float32, (H,))
+    nparts, stride, bcode = 1, 0, F32
+    if branch is not None:
+        nparts, stride = _parts_of(branch, n, H, "norm branch")
+        bcode = _code(branch)
+        if branch_bias is not None:
+            _need(branch_bias, "branch bias", torch.float32, (H,))
+    elif mix is not None or out_weights is not None:
+        raise KernelError("streams_norm: mixing numbers without a branch to add")
+    if mix is not None:
+        _need(mix, "stream mix", torch.float32, (S, S))
+    for t, name in ((out_weights, "stream out weights"), (read, "stream read weights")):
+        if t is not None:
+            _need(t, name, torch.float32, (S,))
+    n_out = n
+    if rows is not None:
+        _need(rows, "norm rows", torch.int32, (None,))
+        n_out = rows.shape[0]
+    _need(out, "norm out", shape=(n_out, H))
+    _check(_fn("norms", "cpmcu_streams_norm")(
+        _p(x), c_long(n * H), c_int(S), _p(branch), c_int(bcode), c_int(nparts), c_long(stride),
+        _p(branch_bias if branch is not None else None), c_float(branch_scale), _p(mix), _p(out_weights), _p(read),
+        c_int(1 if rms else 0), _p(weight), c_float(eps), _p(out), c_int(_code(out)), _p(rows), c_int(n_out), c_int(H),
+        _stream()))
+
+
+def pair_norm_mean(a: torch.Tensor, a_bias: Optional[torch.Tensor], b: torch.Tensor, b_bias: Optional[torch.Tensor],
+                   wa: torch.Tensor, wb: torch.Tensor, eps: float, out: torch.Tensor):
+    """out = (a / rms(a) * wa + b / rms(b) * wb) / 2 row by row in float, rms(v) = sqrt(mean(v^2) + eps): the
+    results of two mixers side by side.  a and b [n, H] or float partial sums [P, n, H], each with an optional
+    bias float32 [H] still to be added."""
+    _need(out, "pair out", torch.float32, (None, None))
+    n, H = out.shape
+    ap, astr = _parts_of(a, n, H, "pair first branch")
+    bp, bstr = _parts_of(b, n, H, "pair second branch")
+    for t, name in ((wa, "first weight"), (wb, "second weight"), (a_bias, "first bias"), (b_bias, "second bias")):
+        if t is not None:
+            _need(t, f"pair {name}", torch.float32, (H,))
+    _check(_fn("norms", "cpmcu_pair_norm_mean")(_p(a), c_int(_code(a)), c_int(ap), c_long(astr), _p(a_bias), _p(b),
+                                                c_int(_code(b)), c_int(bp), c_long(bstr), _p(b_bias), _p(wa), _p(wb),
+                                                c_float(eps), _p(out), c_int(n), c_int(H), _stream()))
+
+
+def sigmoid_gate(a: torch.Tensor, gate: torch.Tensor, out: torch.Tensor):
+    """out = a * sigmoid(gate) element by element; gate may be a column slice of a wider projection."""
+    _need(a, "gate input", shape=(None, None))
+    n, W = a.shape
+    ldg = _ld(gate, "gate")
+    if gate.dtype != a.dtype or tuple(gate.shape) != (n, W):
+        raise KernelError(f"sigmoid_gate: gate {gate.dtype} {tuple(gate.shape)}, expected {a.dtype} {(n, W)}")
+    _need(out, "gate out", a.dtype, (n, W))
+    _check(_fn("norms", "cpmcu_sigmoid_gate")(_p(a), _p(gate), c_long(ldg), _p(out), c_int(_code(a)), c_int(n), c_int(W),
+                                              _stream()))
+
+
+def softcap(logits: torch.Tensor, cap: float):
+    """logits <- cap * tanh(logits / cap), in place (float32)."""
+    _need(logits, "softcap logits", torch.float32)
+    if not cap > 0:
+        raise KernelError(f"softcap: a cap of {cap}")
+    _check(_fn("core", "cpmcu_softcap")(_p(logits), c_long(logits.numel()), c_float(cap), _stream()))
+
+
+def delta_scan(qkv: torch.Tensor, gates: torch.Tensor, a_off: int, b_off: int, dt_bias: torch.Tensor,
+               A_log: torch.Tensor, state: torch.Tensor, y: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor,
+               heads: int, kv_heads: int, dk: int, dv: int, q_scale: float, write_state: bool = True):
+    """The gated delta rule over each sequence's tokens, in float.  qkv float32 [n, 2*kv_heads*dk + heads*dv] =
+    [q | k | v]; gates [n, W] holds the raw decay projection at columns a_off.. and the raw beta projection at
+    b_off.. (heads each).  Per head (its q, k from head h // (heads/kv_heads)): q, k made unit vectors
+    (x / sqrt(sum x^2 + 1e-6)), q times q_scale; beta = sigmoid(b); g = exp(-exp(A_log) softplus(a + dt_bias));
+    S <- g S; u = beta (v - S^T k); S <- S + k u^T; y = S^T q.  state float32 [slots, heads, dv, dk]; y float32
+    [n, heads*dv]."""
+    _need(qkv, "delta inputs", torch.float32, (None, 2 * kv_heads * dk + heads * dv))
+    n = qkv.shape[0]
+    ldg = _ld(gates, "delta gates")
+    if gates.shape[0] != n or min(a_off, b_off) < 0 or max(a_off, b_off) + heads > gates.shape[1]:
+        raise KernelError(f"delta_scan: gate columns {a_off}, {b_off} (+{heads}) lie beyond rows of {tuple(gates.shape)}")
+    _need(dt_bias, "delta dt_bias", torch.float32, (heads,))
+    _need(A_log, "delta A_log", torch.float32, (heads,))
+    _need(state, "delta state", torch.float32, (None, heads, dv, dk))
+    _need(y, "delta out", torch.float32, (n, heads * dv))
+    _need(cu_q, "delta sequence starts", torch.int32, (None,))
+    B = cu_q.shape[0] - 1
+    _need(seq_slot, "delta sequence slots", torch.int32, (B,))
+    _check(_fn("delta", "cpmcu_delta_scan")(_p(qkv), c_long(qkv.shape[1]), _p(gates), c_long(ldg), c_int(_code(gates)),
+                                            c_long(a_off), c_long(b_off), _p(dt_bias), _p(A_log), _p(state), _p(y),
+                                            _p(cu_q), _p(seq_slot), c_int(B), c_int(heads), c_int(kv_heads), c_int(dk),
+                                            c_int(dv), c_float(q_scale), c_int(1 if write_state else 0), _stream()))
+
+
+def diff_qkv_store(src: torch.Tensor, q_out: torch.Tensor, heads: int, kv_heads: int, dk: int, dv: int,
+                   temp_coef: float, temp_every: int, positions: torch.Tensor, tok_slot: torch.Tensor,
+                   kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
+                   page_size: int, write_kv: bool = True):
+    """Between projection and attention of a layer with two score maps a head: a row of src (float32 or q_out's
+    type) is [q: heads*2*dk | k: kv_heads*2*dk | v: kv_heads*dv], q and k head by head as [map 1 | map 2].  q times
+    1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) (temp_every 0: times 1) goes to q_out [n, 2*heads*dk] in
+    the order (kv head, map, head of the group); k into the key pages as 2*kv_heads heads, v into the value pages
+    as kv_heads heads."""
+    ld = _ld(src, "diff qkv")
+    n = src.shape[0]
+    if src.shape[1] < 2 * heads * dk + ((2 * kv_heads * dk + kv_heads * dv) if write_kv else 0):
+        raise KernelError(f"diff_qkv_store: rows of {src.shape[1]} too short")
+    _need(q_out, "diff q_out", shape=(n, 2 * heads * dk))
+    _need(positions, "diff positions", torch.int32, (n,))
+    tw = pk = pv = 0
+    if write_kv:
+        _need(tok_slot, "diff token slots", torch.int32, (n,))
+        _need(page_table, "diff page table", torch.int32, (None, None))
+        _need(kpool, "diff key pool", q_out.dtype, (None, page_size, None))
+        _need(vpool, "diff value pool", q_out.dtype, (kpool.shape[0], page_size, None))
+        if kpool.shape[2] % (2 * kv_heads) or vpool.shape[2] % kv_heads:
+            raise KernelError(f"diff_qkv_store: pools of {kpool.shape[2]} / {vpool.shape[2]} features")
+        tw, pk, pv = page_table.shape[1], kpool.shape[2] // (2 * kv_heads), vpool.shape[2] // kv_heads
+    _check(_fn("attention_general", "cpmcu_diff_qkv_store")(
+        _p(src), c_long(ld), c_int(_code(src)), _p(q_out), c_int(_code(q_out)), c_int(n), c_int(heads), c_int(kv_heads),
+        c_int(dk), c_int(dv), c_float(temp_coef), c_int(temp_every), _p(positions), _p(tok_slot),
+        _p(kpool if write_kv else None), _p(vpool if write_kv else None), _p(page_table if write_kv else None),
+        c_int(tw), c_int(page_size), c_int(pk), c_int(pv), c_int(1 if write_kv else 0), _stream()))
+
+
+def diff_combine(a: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, dv: int, lam: float, eps: float,
+                 post: float):
+    """out[t, h] = o / sqrt(mean(o^2) + eps) * post with o = a1 - lam * a2, the two maps' attention outputs of head
+    h; a [n, 2*heads*dv] in the order (kv head, map, head of the group), out [n, heads*dv]."""
+    _need(a, "diff maps", shape=(None, 2 * heads * dv))
+    n = a.shape[0]
+    _need(out, "diff out", a.dtype, (n, heads * dv))
+    _check(_fn("attention_general", "cpmcu_diff_combine")(_p(a), _p(out), c_int(_code(a)), c_int(n), c_int(heads),
+                                                          c_int(kv_heads), c_int(dv), c_float(lam), c_float(eps),
+                                                          c_float(post), _stream()))
 
 
 MOE_MAX_EXPERTS = 1024
@@ -918,11 +1097,18 @@ def latent_store(proj: torch.Tensor, q_out: torch.Tensor, nh: int, dim: int, rot
         c_int(tw), c_int(page_size), c_int(pk), c_int(pv), c_int(1 if write_cache else 0), _stream()))
 
 
+def _value_heads(nkv: int, v_share: int) -> int:
+    if v_share < 1 or nkv % v_share:
+        raise KernelError(f"attention: {nkv} key heads do not share values in runs of {v_share}")
+    return nkv // v_share
+
+
 def attention_general(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk: int, hdv: int, scale: float,
                       kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
                       positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0, window: int = 0,
-                      keep_first: int = 0, sink: Optional[torch.Tensor] = None):
+                      keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1):
     """Causal attention with key size hdk and value size hdv of their own (plain kernel, both element types).
+    v_share: runs of that many neighbouring key heads read one value head (the value pool holds nkv / v_share heads).
     The cache may hold heads padded to a multiple of 16 features.  chunk > 0: the query at position p sees only
     keys j <= p with j // chunk == p // chunk.  window > 0: only keys with p - j < window, and the sequence's
     first keep_first keys.  sink (float32 [nh]): exp(sink[h]) joins the softmax's denominator as a term without
@@ -934,17 +1120,18 @@ def attention_general(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk
     _need(out, "attention out", q.dtype, (n, nh * hdv))
     _need(kpool, "attention key pool", q.dtype, (None, page_size, None))
     _need(vpool, "attention value pool", q.dtype, (kpool.shape[0], page_size, None))
-    if kpool.shape[2] % nkv or vpool.shape[2] % nkv:
-        raise KernelError(f"attention_general: pools of {kpool.shape[2]} / {vpool.shape[2]} features do not hold {nkv} heads")
+    nvh = _value_heads(nkv, v_share)
+    if kpool.shape[2] % nkv or vpool.shape[2] % nvh:
+        raise KernelError(f"attention_general: pools of {kpool.shape[2]} / {vpool.shape[2]} features do not hold {nkv} / {nvh} heads")
     _need(page_table, "attention page table", torch.int32, (None, None))
     _need(positions, "attention positions", torch.int32, (n,))
     _need(tok_slot, "attention token slots", torch.int32, (n,))
     _check(_fn("attention_general", "cpmcu_attention_general")(
         _p(q), _p(out), c_int(_code(q)), c_int(n), c_int(nh), c_int(nkv), c_int(hdk), c_int(hdv),
-        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nkv), c_float(scale), c_int(chunk), c_int(window),
+        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nvh), c_float(scale), c_int(chunk), c_int(window),
         c_int(keep_first), _p(sink), _p(kpool),
         _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
-        _stream()))
+        c_int(v_share), _stream()))
 
 
 def gemm_heads(x: torch.Tensor, x_off: int, x_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_off: int,
@@ -1142,8 +1329,9 @@ def proj_add_norm(a: torch.Tensor, w: "TiledWeight", alpha: float, x: torch.Tens
                                              c_float(alpha), _p(x), _p(weight), _p(out), _p(sums), _stream()))
 
 
-def gated_strip(x: torch.Tensor, w: "TiledWeight", out: torch.Tensor, row_scale: Optional[RowScale] = None):
-    """out = silu(x . Wg^T) * (x . Wu^T) for a step of at most 16 tokens, w tiled with the gate rows first (a
+def gated_strip(x: torch.Tensor, w: "TiledWeight", out: torch.Tensor, row_scale: Optional[RowScale] = None,
+                activation: str = "silu"):
+    """out = act(x . Wg^T) * (x . Wu^T) (act as in silu_mul) for a step of at most 16 tokens, w tiled with the gate rows first (a
     multiple of 16 of them); out bfloat16 [n, N/2].  With row_scale as in gemm_skinny."""
     _need(x, "gated x", torch.bfloat16, (None, None))
     n, K = x.shape
@@ -1155,15 +1343,16 @@ def gated_strip(x: torch.Tensor, w: "TiledWeight", out: torch.Tensor, row_scale:
     _check(_fn("qkv", "cpmcu_gated_strip")(_p(x), c_long(K), _p(w.data), c_int(n), c_int(w.N // 2), c_int(K), _p(out),
                                            _p(row_scale.sums if row_scale is not None else None),
                                            c_int(row_scale.sums.shape[1] if row_scale is not None else 0),
-                                           c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
+                                           c_float(row_scale.eps if row_scale is not None else 0.0),
+                                           c_int(_act(activation)), _stream()))
 
 
 def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain",
-                row_scale: Optional[RowScale] = None):
+                row_scale: Optional[RowScale] = None, activation: str = "silu"):
     """bf16 product for at most 64 rows of x on the matrix cores, streaming w once; w is [N, K] as in the
     checkpoint or a TiledWeight.
     mode 'plain': out [m,N] float32 or bfloat16; 'partial': out float32 [S,m,N], S slices of K to be summed by
-    the consumer; 'gated': w holds gate rows then up rows, out bfloat16 [m,N/2] = silu(gate) * up.
+    the consumer; 'gated': w holds gate rows then up rows, out bfloat16 [m,N/2] = act(gate) * up (act as in silu_mul).
     With row_scale, x is the x * w of add_norm_columns: the rows of the product are multiplied by the norm's
     factor (before the gate's nonlinearity)."""
     _need(x, "gemm x", torch.bfloat16, (None, None))
@@ -1195,7 +1384,8 @@ def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode:
                                             c_int(ksplit), c_float(alpha), c_int(1 if tiled else 0),
                                             _p(row_scale.sums if row_scale is not None else None),
                                             c_int(row_scale.sums.shape[1] if row_scale is not None else 0),
-                                            c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
+                                            c_float(row_scale.eps if row_scale is not None else 0.0),
+                                            c_int(_act(activation)), _stream()))
 
 
 SKINNY_MAX_ROWS = 64
@@ -1309,7 +1499,7 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
                            positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0, n_splits: int = 1,
                            part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                            tiles: Optional[torch.Tensor] = None, tokens_per_tile: int = 1, window: int = 0,
-                           keep_first: int = 0, sink: Optional[torch.Tensor] = None):
+                           keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1):
     """attention_general in bf16 on the matrix cores (key size a multiple of 8 up to 1024, value size up to 512).
     With n_splits > 1 every token's visible keys are shared among n_splits workgroups and merged afterwards;
     part_o float32 [n, nh, n_splits, hdv] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
@@ -1321,8 +1511,9 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
     _need(out, "attention out", torch.bfloat16, (n, nh * hdv))
     _need(kpool, "attention key pool", torch.bfloat16, (None, page_size, None))
     _need(vpool, "attention value pool", torch.bfloat16, (kpool.shape[0], page_size, None))
-    if kpool.shape[2] % nkv or vpool.shape[2] % nkv:
-        raise KernelError(f"attention_general: pools of {kpool.shape[2]} / {vpool.shape[2]} features do not hold {nkv} heads")
+    nvh = _value_heads(nkv, v_share)
+    if kpool.shape[2] % nkv or vpool.shape[2] % nvh:
+        raise KernelError(f"attention_general: pools of {kpool.shape[2]} / {vpool.shape[2]} features do not hold {nkv} / {nvh} heads")
     _need(page_table, "attention page table", torch.int32, (None, None))
     _need(positions, "attention positions", torch.int32, (n,))
     _need(tok_slot, "attention token slots", torch.int32, (n,))
@@ -1335,10 +1526,11 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
         _need(sink, "attention sink", torch.float32, (nh,))
     _check(_fn("attention_general", "cpmcu_attention_general_mfma")(
         _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hdk), c_int(hdv),
-        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nkv), c_float(scale), c_int(chunk), c_int(window),
+        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nvh), c_float(scale), c_int(chunk), c_int(window),
         c_int(keep_first), _p(sink), _p(kpool), _p(vpool),
         _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot), c_int(n_splits),
-        _p(tiles), c_int(tiles.shape[0] if tiles is not None else 0), c_int(tokens_per_tile), _stream()))
+        _p(tiles), c_int(tiles.shape[0] if tiles is not None else 0), c_int(tokens_per_tile), c_int(v_share),
+        _stream()))
 
 
 def attention_general_tokens_per_tile(n_tokens: int, nh: int, nkv: int, pool_hdv: int) -> int:
@@ -1364,11 +1556,13 @@ def reserve_attention_general(ws, dtype, nh: int, nkv: int, hdv: int, pool_hdv: 
 
 
 def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx, chunk: int = 0,
-                  window: int = 0, keep_first: int = 0, sink: Optional[torch.Tensor] = None):
+                  window: int = 0, keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1):
     """Attention with key and value sizes of their own and an optional mask (chunks, or a sliding window with kept
-    first tokens) and softmax sink, with the kernel that suits the step; writes ``out`` [n, nh*hdv]."""
+    first tokens) and softmax sink, with the kernel that suits the step; writes ``out`` [n, nh*hdv].  v_share:
+    runs of that many neighbouring key heads read one value head."""
+    pool_hdv = vpool.shape[2] // _value_heads(nkv, v_share)
     if (hdk == hdv and chunk == 0 and window == 0 and sink is None and hdk <= 256 and hdk % 16 == 0
-            and kpool.shape[2] == nkv * hdk):
+            and kpool.shape[2] == nkv * hdk and v_share == 1):
         attention(q, out, nh, nkv, hdk, scale, kpool, vpool, page_table, page_size, ctx)
         return
     if attention_general_mfma_ok(q, hdk, hdv, page_size):
@@ -1378,21 +1572,21 @@ def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, pa
             keys = min(keys, chunk)
         if window:
             keys = min(keys, window + keep_first)
-        splits = attention_general_splits(n, nkv, nh // nkv, vpool.shape[2] // nkv, keys) if ctx.single_token else 1
+        splits = attention_general_splits(n, nkv, nh // nkv, pool_hdv, keys) if ctx.single_token else 1
         part_o = part_ml = None
         if splits > 1:
             part_o = ctx.ws.get("attn.gpart_o", (n, nh, splits, hdv), torch.float32)
             part_ml = ctx.ws.get("attn.gpart_ml", (n, nh, splits, 2), torch.float32)
         tiles, tpt = None, 1
         if not ctx.single_token:
-            tpt = attention_general_tokens_per_tile(n, nh, nkv, vpool.shape[2] // nkv)
+            tpt = attention_general_tokens_per_tile(n, nh, nkv, pool_hdv)
             if tpt > 1:
                 key = ("prefill_tiles", tpt)
                 tiles = ctx.extras.get(key)
                 if tiles is None:
                     tiles = ctx.extras[key] = prefill_tiles(ctx.q_lens, tpt, q.device)
         attention_general_mfma(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
-                               ctx.tok_slot, chunk, splits, part_o, part_ml, tiles, tpt, window, keep_first, sink)
+                               ctx.tok_slot, chunk, splits, part_o, part_ml, tiles, tpt, window, keep_first, sink, v_share)
         return
     attention_general(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
-                      ctx.tok_slot, chunk, window, keep_first, sink)
+                      ctx.tok_slot, chunk, window, keep_first, sink, v_share)

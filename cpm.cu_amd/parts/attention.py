@@ -236,15 +236,22 @@ class GeneralAttention(Mixer):
       'q_norm', 'k_norm'   weights of dk numbers, shared by the heads: q and k heads are divided by their root mean
                            square (``norm_eps`` inside the root) and multiplied by them before the rotation;
       'sink'               one number a head: exp(sink) joins the softmax's denominator as a term that has no key,
-                           no value and no scale.
+                           no value and no scale;
+      'gate'               an output gate: the heads side by side are multiplied element by element with
+                           sigmoid(W_gate h) before the output projection (its rows ride in the q/k/v product).
+    ``unit_norm_after_rotation``: q and k heads are divided by their root mean square (``norm_eps`` inside the
+    root, no weight) after the rotation.
     Without 'v' the values are the keys as projected (with their bias, before norm and rotation): value_dim
     must equal key_dim."""
 
     def __init__(self, names: Mapping[str, str], hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int,
                  value_dim: int, position: Optional[PositionEncoding], scale: float, mask_chunk: Optional[int] = None,
-                 mask_window: Optional[int] = None, mask_keep_first: int = 0, norm_eps: float = 0.0):
+                 mask_window: Optional[int] = None, mask_keep_first: int = 0, norm_eps: float = 0.0,
+                 unit_norm_after_rotation: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if unit_norm_after_rotation and (names.get("q_norm") or names.get("k_norm")):
+            raise ValueError("attention: a norm after the rotation has no weights")
         if key_dim > 1024 or value_dim > 1024:
             raise ValueError(f"attention: key size {key_dim} / value size {value_dim} exceed the kernel's 1024")
         if mask_chunk is not None and mask_chunk <= 0:
@@ -267,11 +274,18 @@ class GeneralAttention(Mixer):
         if not self.values_are_keys:
             stacked.append((self.names["v"], num_kv_heads * value_dim))
             biases.append(self.names.get("v_bias"))
+        self.norm_after = bool(unit_norm_after_rotation)
+        self.gate_off = None
+        if self.names.get("gate"):
+            self.gate_off = sum(r for _, r in stacked)
+            stacked.append((self.names["gate"], num_heads * value_dim))
+            biases.append(None)
         self.qkv = Linear(stacked, hidden_size, bias_names=biases if any(biases) else None)
         self.o = Linear([(self.names["out"], hidden_size)], num_heads * value_dim,
                         bias_names=[self.names["out_bias"]] if self.names.get("out_bias") else None)
         # what the plain rotate-and-store kernel does not do
-        self._extras = bool(any(biases) or self.names.get("q_norm") or self.names.get("k_norm") or self.values_are_keys)
+        self._extras = bool(any(biases) or self.names.get("q_norm") or self.names.get("k_norm") or self.values_are_keys
+                            or self.norm_after)
 
     def parts(self) -> List[Part]:
         return [self.qkv, self.o] + ([self.position] if self.position is not None else [])
@@ -311,13 +325,14 @@ class GeneralAttention(Mixer):
         if rd > dk:
             raise ValueError(f"attention: the rotation covers {rd} features, a head has {dk}")
         with ctx.timed("attn_qkv_rope"):
-            qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * dk)
+            qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if (writes_cache or self.gate_off is not None) else nh * dk)
             q = ctx.ws.get("attn.q", (n, nh * dk), self.rt.dtype)
             if self._extras:
                 ops.qkv_norm_rotate_store(qkv, q, nh, nkv, dk, dv, rd, ctx.positions, ctx.tok_slot, inv_freq, mag,
                                           cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
                                           write_kv=writes_cache, bias=self.qkv.bias, q_norm=self.q_norm,
-                                          k_norm=self.k_norm, eps=self.norm_eps, values_from_keys=self.values_are_keys)
+                                          k_norm=self.k_norm, eps=self.norm_eps, values_from_keys=self.values_are_keys,
+                                          norm_after=self.norm_after)
             else:
                 ops.qkv_rotate_store(qkv, q, nh, nkv, dk, dv, rd, ctx.positions, ctx.tok_slot, inv_freq, mag,
                                      cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
@@ -327,6 +342,11 @@ class GeneralAttention(Mixer):
             ops.attention_any(q, out, nh, nkv, dk, dv, self.scale, cache.streams["k"], cache.streams["v"],
                               cache.page_table, cache.page_size, ctx, chunk=self.chunk, window=self.window,
                               keep_first=self.keep_first, sink=self.sink)
+        if self.gate_off is not None:
+            with ctx.timed("attn_gate"):
+                gated = ctx.ws.get("attn.gated", (n, nh * dv), self.rt.dtype)
+                ops.sigmoid_gate(out, qkv[:, self.gate_off:self.gate_off + nh * dv], gated)
+                out = gated
         with ctx.timed("attn_o"):
             branch = self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)
         return BiasedBranch(branch, self.o.bias, ctx, "attn.o") if self.o.bias is not None else branch

@@ -190,6 +190,22 @@ class BiasedBranch:
         return self._value
 
 
+class StreamsBranch:
+    """A sub-layer's result that joins a residual of several streams (hyper-connections): all streams at once,
+    x_t <- sum_s ``mix``[s, t] x_s + ``out``[t] * ``branch`` (mix float32 [S, S] indexed [from, to], out float32
+    [S]).  ``branch`` is a tensor [n, H], float partial sums [P, n, H] or a BiasedBranch.  It is left pending like
+    every branch and added by the norm that follows (``Norm.forward_streams``)."""
+
+    def __init__(self, branch, mix: torch.Tensor, out: torch.Tensor):
+        self.branch, self.mix, self.out = branch, mix, out
+
+    def pieces(self):
+        """(tensor, bias or None) of the branch."""
+        if isinstance(self.branch, BiasedBranch):
+            return self.branch.branch, self.branch.bias
+        return branch_tensor(self.branch), None
+
+
 def branch_tensor(branch):
     """The branch as a tensor (or None), whatever form it was handed over in."""
     return branch.evaluate() if isinstance(branch, (DeferredBranch, NormedBranch, BiasedBranch)) else branch
@@ -293,6 +309,13 @@ class Norm(Part):
     takes_normed_branch = False
     # True if forward and forward_unscaled accept a BiasedBranch as ``branch``
     takes_biased_branch = False
+
+    def forward_streams(self, x: torch.Tensor, pending: Optional["StreamsBranch"], read: Optional[torch.Tensor],
+                        ctx: StepContext, rows: Optional[torch.Tensor] = None, tag: str = "norm") -> torch.Tensor:
+        """For a residual of several streams x float32 [S, n, H]: add the pending StreamsBranch into the streams
+        (in place, unless ``rows`` selects rows), read u = sum_s read[s] x_s (read float32 [S]; None: the plain
+        sum) and return this norm of u.  A norm that a model with such a residual uses defines it."""
+        raise NotImplementedError(f"{type(self).__name__} does not read a residual of several streams")
 
     def normalize(self, t: torch.Tensor, ctx: StepContext, tag: str = "norm.plain") -> torch.Tensor:
         """The norm of the rows of ``t`` alone, float32 [n, H]: no residual, nothing added (what a branch that

@@ -15,14 +15,17 @@ import torch
 
 from .. import ops
 from .base import (BLOCKS, BiasedBranch, Block, DeferredBranch, FeedForward, Mixer, Norm, NormedBranch, Part,
-                   ResidualStream, StepContext, branch_for, branch_tensor, forward_declares)
+                   ResidualStream, Runtime, StepContext, StreamsBranch, WeightSpec, branch_for, branch_tensor,
+                   forward_declares)
 from .linear import Linear
 
 
 @BLOCKS.register("pre_norm")
 class PreNormBlock(Block):
-    def __init__(self, mixer_norm: Norm, mixer: Mixer, ff_norm: Norm, feed_forward: FeedForward,
-                 residual_scale: float = 1.0):
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ff_norm: Optional[Norm] = None,
+                 feed_forward: Optional[FeedForward] = None, residual_scale: float = 1.0):
+        if (feed_forward is None) != (ff_norm is None):
+            raise ValueError("pre_norm: a feed-forward comes with its norm, or neither is given")
         self.mixer_norm = mixer_norm
         self.mixer = mixer
         self.ff_norm = ff_norm
@@ -32,10 +35,10 @@ class PreNormBlock(Block):
         # defines ``forward`` says so itself, so a subclass with a forward of its own is asked only if it
         # declares the same
         self._mixer_defers = forward_declares(mixer, "can_defer_last")
-        self._ff_defers = forward_declares(feed_forward, "can_defer_last")
+        self._ff_defers = feed_forward is not None and forward_declares(feed_forward, "can_defer_last")
 
     def parts(self) -> List[Part]:
-        return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
+        return [self.mixer_norm, self.mixer] + ([self.ff_norm, self.feed_forward] if self.feed_forward is not None else [])
 
     @staticmethod
     def _normed(norm: Norm, deferred: bool, x, branch, branch_scale, ctx):
@@ -74,8 +77,11 @@ class PreNormBlock(Block):
         # (src/model/minicpm4/minicpm4_layer.cuh:46-83); the parts inside time their own kernels by class
         with ctx.timed("attn"):
             a = self._mix(stream, ctx, cache, writes_cache)
-        with ctx.timed("ffn"):
-            stream.pending = self._feed(stream, a, ctx)
+        if self.feed_forward is None:           # a layer without a feed-forward leaves its mixer's branch pending
+            stream.pending = a
+        else:
+            with ctx.timed("ffn"):
+                stream.pending = self._feed(stream, a, ctx)
         stream.pending_scale = self.residual_scale
 
 
@@ -157,4 +163,58 @@ class ParallelGatedBlock(Block):
             out = ctx.ws.get("block.gated", (h.shape[0], self.hidden_size), torch.float32)
             ops.gated_branches(g, self.gates.bias, a, a_bias, f, f_bias, out)
         stream.pending = out
+        stream.pending_scale = 1.0
+
+
+@BLOCKS.register("hyper_connections")
+class HyperConnectionBlock(Block):
+    """Pre-norm sub-layers over a residual of S streams (hyper-connections).  Sub-layer q (1: mixer, 2:
+    feed-forward, which a layer may lack) has numbers in[S], out[S] and mix[S, S] of its own:
+
+        u = sum_s in[s] x_s;   y = sub(norm(u));   x_t <- sum_s mix[s, t] x_s + out[t] * y    (all t at once)
+
+    The result is left pending as a StreamsBranch and added by the norm that follows, which reads the streams with
+    the next sub-layer's ``in`` in the same pass (Norm.forward_streams).
+    ``names``: for each sub-layer the checkpoint tensors (in, out, mix)."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, streams: int, names: List[tuple], ff_norm: Optional[Norm] = None,
+                 feed_forward: Optional[FeedForward] = None):
+        if (feed_forward is None) != (ff_norm is None):
+            raise ValueError("hyper_connections: a feed-forward comes with its norm, or neither is given")
+        if len(names) != (2 if feed_forward is not None else 1):
+            raise ValueError("hyper_connections: tensors (in, out, mix) for every sub-layer")
+        if streams < 1:
+            raise ValueError(f"hyper_connections: {streams} streams")
+        self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward = mixer_norm, mixer, ff_norm, feed_forward
+        self.streams, self.names = int(streams), [tuple(t) for t in names]
+
+    def parts(self) -> List[Part]:
+        return [self.mixer_norm, self.mixer] + ([self.ff_norm, self.feed_forward] if self.feed_forward is not None else [])
+
+    def weight_specs(self) -> List[WeightSpec]:
+        S, specs = self.streams, []
+        for read, out, mix in self.names:
+            specs += [WeightSpec(read, (S,), "stream_read"), WeightSpec(out, (S,), "norm"), WeightSpec(mix, (S, S), "stream_mix")]
+        return specs
+
+    def bind(self, tensors, rt: Runtime):
+        f = lambda name: tensors[name].to(torch.float32).contiguous()
+        self.numbers = [(f(read), f(out), f(mix)) for read, out, mix in self.names]
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True):
+        x = stream.x
+        if x.dim() != 3 or x.shape[0] != self.streams:
+            raise ValueError(f"hyper_connections: the residual has shape {tuple(x.shape)}, {self.streams} streams expected")
+        read, out, mix = self.numbers[0]
+        with ctx.timed("attn"):
+            with ctx.timed("norm"):
+                h = self.mixer_norm.forward_streams(x, stream.take_pending(), read, ctx, tag="block.h")
+            pending = StreamsBranch(self.mixer.forward(h, ctx, cache, writes_cache), mix, out)
+        if self.feed_forward is not None:
+            read, out, mix = self.numbers[1]
+            with ctx.timed("ffn"):
+                with ctx.timed("norm"):
+                    h = self.ff_norm.forward_streams(x, pending, read, ctx, tag="block.h")
+                pending = StreamsBranch(self.feed_forward.forward(h, ctx), mix, out)
+        stream.pending = pending
         stream.pending_scale = 1.0

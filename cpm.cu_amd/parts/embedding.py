@@ -36,7 +36,11 @@ class TokenEmbedding(Part):
 
 class LMHead(Part):
     def __init__(self, name: str, vocab_size: int, hidden_size: int, scale: float = 1.0,
-                 tied_to: Optional[TokenEmbedding] = None):
+                 tied_to: Optional[TokenEmbedding] = None, softcap: Optional[float] = None):
+        """``softcap`` c: the logits leave as c * tanh(logits / c)."""
+        if softcap is not None and not softcap > 0:
+            raise ValueError(f"head: a logit cap of {softcap}")
+        self.softcap = float(softcap) if softcap is not None else None
         self.name = name
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
@@ -68,4 +72,6 @@ class LMHead(Part):
             self.tiled = ops.TiledWeight(w)
         logits = ctx.ws.get("logits", (y.shape[0], self.vocab_size), torch.float32)
         ops.linear(y, w, logits, self.scale, w_tiled=self.tiled)
+        if self.softcap is not None:
+            ops.softcap(logits, self.softcap)
         return logits

@@ -1,4 +1,4 @@
-"""SiLU-gated feed-forward: down( silu(x Wg^T) * (x Wu^T) ).
+"""Gated feed-forward: down( act(x Wg^T) * (x Wu^T) ), act = SiLU (or the tanh form of GELU).
 
 gate and up are one stacked product, gate rows first (src/model/ffn.cuh:31-59,
 77-84); silu(g) * u in float (src/model/activation.cuh:6-18).
@@ -14,11 +14,17 @@ from .base import FEED_FORWARDS, DeferredBranch, FeedForward, Part, Runtime, Ste
 from .linear import Linear
 
 
+@FEED_FORWARDS.register("gated")
 @FEED_FORWARDS.register("gated_silu")
 class GatedFFN(FeedForward):
-    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, names: Optional[Mapping[str, str]] = None):
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, names: Optional[Mapping[str, str]] = None,
+                 activation: str = "silu"):
         """``names``: the checkpoint tensors for 'gate', 'up', 'down' behind the prefix (default: the MiniCPM
-        checkpoint's gate_proj.weight, up_proj.weight, down_proj.weight)."""
+        checkpoint's gate_proj.weight, up_proj.weight, down_proj.weight).  ``activation``: the gate's
+        nonlinearity, 'silu' or 'gelu_tanh' (0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))))."""
+        if activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"feed-forward: gate nonlinearity '{activation}' (known: {sorted(ops.GATE_ACTIVATIONS)})")
+        self.activation = activation
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         names = names or {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
@@ -36,7 +42,7 @@ class GatedFFN(FeedForward):
 
     def forward(self, h: torch.Tensor, ctx: StepContext, row_scale=None, defer_last: bool = False):
         with ctx.timed("ffn_gate_up"):
-            act = self.gate_up.forward_gated(h, ctx, "ffn.gate_up", row_scale=row_scale)
+            act = self.gate_up.forward_gated(h, ctx, "ffn.gate_up", row_scale=row_scale, activation=self.activation)
         if defer_last and self.down.defers(act):
             return DeferredBranch(self.down, act, ctx, "ffn.down")
         with ctx.timed("ffn_down"):

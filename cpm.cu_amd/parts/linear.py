@@ -95,19 +95,21 @@ class Linear(Part):
         """Whether forward_gated, for n rows, runs the kernel that can finish a norm (ops.RowScale)."""
         return self._gated_skinny(n, self.rt.dtype)
 
-    def forward_gated(self, x: torch.Tensor, ctx: StepContext, tag: str, row_scale=None) -> torch.Tensor:
-        """For a weight of gate rows stacked on up rows: silu(x Wg^T) * (x Wu^T), [n, out/2]."""
+    def forward_gated(self, x: torch.Tensor, ctx: StepContext, tag: str, row_scale=None,
+                      activation: str = "silu") -> torch.Tensor:
+        """For a weight of gate rows stacked on up rows: act(x Wg^T) * (x Wu^T), [n, out/2]; act is SiLU or
+        another of ops.GATE_ACTIVATIONS."""
         n, half = x.shape[0], self.out_features // 2
         act = ctx.ws.get(tag + ".act", (n, half), x.dtype)
         if (n <= ops.STRIP_ROWS and x.dtype == torch.bfloat16 and self.tiled is not None and half % 16 == 0
                 and self.in_features % 8 == 0):
-            ops.gated_strip(x, self.tiled, act, row_scale=row_scale)      # a strip of columns a workgroup
+            ops.gated_strip(x, self.tiled, act, row_scale=row_scale, activation=activation)   # a strip of columns a workgroup
         elif self._gated_skinny(n, x.dtype):
             ops.gemm_skinny(x, self.tiled if self.tiled is not None else self.weight, act, mode="gated",
-                            row_scale=row_scale)
+                            row_scale=row_scale, activation=activation)
         else:
             if row_scale is not None:
                 raise ValueError("forward_gated: a row scale needs the few-rows kernel (gated_takes_row_scale)")
             gu = self.forward(x, ctx, tag)
-            ops.silu_mul(gu, act)
+            ops.silu_mul(gu, act, activation)
         return act

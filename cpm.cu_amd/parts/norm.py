@@ -11,7 +11,8 @@ from typing import List, Mapping, Optional
 import torch
 
 from .. import ops
-from .base import NORMS, DeferredBranch, Norm, NormedBranch, Runtime, StepContext, WeightSpec, branch_tensor
+from .base import (NORMS, BiasedBranch, DeferredBranch, Norm, NormedBranch, Runtime, StepContext, StreamsBranch, WeightSpec,
+                   branch_tensor)
 
 
 @NORMS.register("rms_norm")
@@ -59,6 +60,9 @@ class RMSNorm(Norm):
         ops.add_rms_norm(x, branch, branch_scale, self.weight, self.eps, out, rows)
         return out
 
+    def forward_streams(self, x, pending, read, ctx: StepContext, rows=None, tag="norm"):
+        return _streams_norm(self, x, pending, read, ctx, rows, tag, rms=True)
+
     def forward_unscaled(self, x, branch, branch_scale, ctx: StepContext, tag="norm"):
         # decode steps: a row a workgroup leaves most of the chip idle, so the work is cut by columns and the
         # row factor rsqrt(mean(x^2) + eps) is left to the product that follows
@@ -81,3 +85,47 @@ class RMSNorm(Norm):
         sums = ctx.ws.get(tag + ".sums", (n, ops.norm_slices(self.hidden_size)), torch.float32)
         ops.add_norm_columns(x, branch, branch_scale, self.weight, out, sums)
         return out, ops.RowScale(sums, self.eps)
+
+
+def _streams_norm(norm, x, pending: Optional[StreamsBranch], read, ctx: StepContext, rows, tag: str, rms: bool):
+    n_out = x.shape[-2] if rows is None else rows.shape[0]
+    out = ctx.ws.get(tag, (n_out, norm.hidden_size), norm.rt.dtype)
+    branch = bias = mix = outw = None
+    if pending is not None:
+        (branch, bias), mix, outw = pending.pieces(), pending.mix, pending.out
+    ops.streams_norm(x, branch, bias, 1.0, mix, outw, read, norm.weight, norm.eps, out, rows, rms=rms)
+    return out
+
+
+@NORMS.register("layer_norm")
+class LayerNorm(Norm):
+    """Layer norm with a weight and no bias: y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w, statistics in
+    float, with the residual add fused in front of it like RMSNorm's; it also reads a residual of several streams."""
+
+    def __init__(self, name: str, hidden_size: int, eps: float):
+        self.name = name
+        self.hidden_size = hidden_size
+        self.eps = float(eps)
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return [WeightSpec(self.name, (self.hidden_size,), "norm")]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        self.weight = tensors[self.name].to(torch.float32).contiguous()
+        self.rt = rt
+
+    takes_biased_branch = True
+
+    def forward(self, x, branch, branch_scale, ctx: StepContext, rows=None, tag="norm"):
+        n_out = x.shape[0] if rows is None else rows.shape[0]
+        out = ctx.ws.get(tag, (n_out, self.hidden_size), self.rt.dtype)
+        bias = None
+        if isinstance(branch, BiasedBranch):
+            branch, bias = branch.branch, branch.bias
+            if branch_scale != 1.0:
+                raise ValueError("layer_norm: a branch with a pending bias cannot be scaled")
+        ops.streams_norm(x, branch_tensor(branch), bias, branch_scale, None, None, None, self.weight, self.eps, out, rows)
+        return out
+
+    def forward_streams(self, x, pending, read, ctx: StepContext, rows=None, tag="norm"):
+        return _streams_norm(self, x, pending, read, ctx, rows, tag, rms=False)

@@ -86,3 +86,26 @@ class YarnRotaryEncoding(RotaryEncoding):
         hi = min(math.ceil(self._turns_to_feature(self.slow)), self.head_dim - 1)
         ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
         self.inv_freq = (f / self.factor * ramp + f * (1.0 - ramp)).to(torch.float32).to(rt.device)
+
+
+@POSITION_ENCODINGS.register("llama3")
+class Llama3RotaryEncoding(RotaryEncoding):
+    """Rotation of ``head_dim`` features whose slow frequencies are stretched (the frequency scaling of Llama 3.1).
+    With f_i = theta^(-2i/head_dim) and wavelength l_i = 2 pi / f_i: f_i stays where l_i < original / high, becomes
+    f_i / factor where l_i > original / low, and in between is (1 - t) f_i / factor + t f_i with
+    t = (original / l_i - low) / (high - low).  The magnitude stays 1."""
+
+    def __init__(self, head_dim: int, theta: float, factor: float, low: float, high: float, original: float):
+        super().__init__(head_dim, theta)
+        self.factor, self.low, self.high, self.original = float(factor), float(low), float(high), float(original)
+        if self.factor <= 0 or self.high <= self.low or self.original <= 0:
+            raise ValueError(f"llama3 rotation: factor {factor}, low {low}, high {high}, original {original}")
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        i = torch.arange(0, self.head_dim // 2, dtype=torch.float64)
+        f = self.theta ** (-2.0 * i / self.head_dim)
+        wave = 2.0 * math.pi / f
+        t = ((self.original / wave - self.low) / (self.high - self.low)).clamp(0.0, 1.0)
+        blend = (1.0 - t) * f / self.factor + t * f
+        out = torch.where(wave < self.original / self.high, f, torch.where(wave > self.original / self.low, f / self.factor, blend))
+        self.inv_freq = out.to(torch.float32).to(rt.device)

@@ -94,6 +94,20 @@ def _init_log_decay(spec, g, device, dtype, std, norm_std):
     return torch.log(0.05 + 3.95 * u).to(dtype)
 
 
+@register_init_rule("stream_read")
+def _init_stream_read(spec, g, device, dtype, std, norm_std):
+    """1/S + N(0, 0.2): the numbers with which a sub-layer reads a residual of S streams (near their mean)."""
+    t = torch.full(spec.shape, 1.0 / spec.shape[-1], dtype=torch.float32, device=device)
+    return (t + torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * 0.2).to(dtype)
+
+
+@register_init_rule("stream_mix")
+def _init_stream_mix(spec, g, device, dtype, std, norm_std):
+    """identity + N(0, 0.15): the matrix that carries a residual of several streams past a sub-layer."""
+    t = torch.eye(spec.shape[-1], dtype=torch.float32, device=device).expand(spec.shape).clone()
+    return (t + torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * 0.15).to(dtype)
+
+
 @register_init_rule("matrix")
 def _init_matrix(spec, g, device, dtype, std, norm_std):
     """N(0, std)."""
