@@ -172,14 +172,16 @@ def main():
     ap.add_argument("--perf", action="store_true",
                     help="after the timed runs, a few eager steps with the engine's timers on: average ms by kernel "
                          "class (products / attention / selection / norms / head) on stderr and under 'timers'")
-    ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k", "duvulix", "gumodra"],
+    ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k", "duvulix", "gumodra", "sagedra"],
                     help="headline: the 8B shape at batch 8, context 4,096 (the default line); "
                          "small_batch64: the 0.5B shape, 64 unequal prompts through the generation loop; sparse32k: "
                          "the 8B shape with InfLLM-v2 at 32k context; duvulix: four Duvulix layers of a real model's "
                          "sizes (latent attention, chunked attention, Mamba-2, a layer that reads the first one's "
                          "latent cache) beside four MiniCPM4-8B layers of equal width: decode and prefill of both; gumodra: "
                          "four Gumodra layers of a real model's sizes (windowed attention with a sink, mLSTM, dense and "
-                         "routed feed-forwards) beside the four Duvulix layers")
+                         "routed feed-forwards) beside the four Duvulix layers; sagedra: four Sagedra layers of a real model's sizes "
+                         "(differential attention, windowed attention beside a gated delta rule, four residual streams) "
+                         "beside the four Gumodra layers")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path exists)")
@@ -482,6 +484,59 @@ def gumodra_prefill_params(raw):
     return total
 
 
+def config_sagedra():
+    """Four layers of sizes that resemble a real model's: width 4,096 in 4 residual streams; differential attention
+    with 16 heads of two maps each on 4 key heads of 128 and values of 256, 4 convolution taps and a query
+    temperature; pairs of a sliding-window attention (32 heads on 8 kv heads of 128, all features rotated with
+    stretched frequencies, a window of 2,048, an output gate) beside a gated delta rule (32 heads on 16 key heads,
+    128 by 128, 4 taps); GELU-gated feed-forwards of 11,008; a logit cap."""
+    diff = {"heads": 16, "kv_heads": 4, "dim": 128, "vdim": 256, "scale": 128 ** -0.5, "diff": 0.5, "conv": 4,
+            "q_temp": {"coef": 0.1, "every": 1024}}
+    pair = {"left": {"heads": 32, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 1.0,
+                     "rot": {"base": 500000.0, "dims": 128,
+                             "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
+                     "mask": {"size": 2048}},
+            "right": {"heads": 32, "kv_heads": 16, "dim": 128, "vdim": 128, "conv": 4}}
+    dense = {"kind": "dense", "ff": 11008}
+    return {
+        "architecture": "Sagedra", "vocab": 73448, "width": 4096, "norm": {"eps": 1e-5}, "embedding": {"scale": 12.0},
+        "streams": 4, "logit_softcap": 30.0,
+        "layers": [
+            {"type": "attention", "mixer": dict(diff), "mlp": dense},
+            {"type": "parallel", "mixer": dict(pair), "mlp": dense},
+            {"type": "attention", "mixer": dict(diff), "mlp": dense},
+            {"type": "parallel", "mixer": dict(pair), "mlp": dense},
+        ],
+    }
+
+
+def sagedra_step_bytes(raw, esize, batch, context):
+    """Bytes a decode step must move: every matrix once, and per sequence what its mixers read: keys of both maps
+    and the values of all cached tokens (differential attention), keys and values of the window, the delta rule's
+    state read and written, the convolutions' last inputs."""
+    W = raw["width"]
+    weights = raw["vocab"] * W
+    per_seq = 0
+    for layer in raw["layers"]:
+        m = layer["mixer"]
+        if layer["type"] == "attention":
+            qk, v = 2 * m["dim"], m["vdim"]
+            weights += (m["heads"] * (qk + v) + m["kv_heads"] * (qk + v)) * W
+            per_seq += context * m["kv_heads"] * (qk + v) * esize
+            per_seq += 2 * 4 * (m.get("conv", 1) - 1) * (m["heads"] * qk + m["kv_heads"] * (qk + v))
+        else:
+            a, d = m["left"], m["right"]
+            weights += (a["heads"] * (a["dim"] + 2 * a["vdim"]) + a["kv_heads"] * (a["dim"] + a["vdim"])) * W
+            seen = context if not a.get("mask") else min(context, a["mask"]["size"])
+            per_seq += seen * a["kv_heads"] * (a["dim"] + a["vdim"]) * esize
+            hk, hv = d["kv_heads"] * d["dim"], d["heads"] * d["vdim"]
+            weights += (2 * hk + 3 * hv + 2 * d["heads"]) * W
+            per_seq += 2 * 4 * (d["heads"] * d["dim"] * d["vdim"] + (d["conv"] - 1) * (2 * hk + hv))
+        if layer.get("mlp"):
+            weights += 3 * layer["mlp"]["ff"] * W
+    return weights * esize + batch * per_seq, weights
+
+
 def duvulix_scenario(args, dev):
     """Decode and prefill of the Duvulix layer shapes beside the MiniCPM4-8B layer shape (equal width, equal
     number of layers, random weights): one JSON line with both models' figures and their timers by kernel class."""
@@ -492,6 +547,12 @@ def gumodra_scenario(args, dev):
     """The same for the Gumodra layer shapes beside the Duvulix layer shapes (the package's other design of mixed
     attention and recurrent layers; equal width, vocabulary and number of layers)."""
     layer_shapes_scenario(args, dev, "gumodra", "Gumodra", config_gumodra(), ("duvulix", config_duvulix()))
+
+
+def sagedra_scenario(args, dev):
+    """The same for the Sagedra layer shapes beside the Gumodra layer shapes (the package's closest design: windowed
+    attention beside a matrix-state recurrence; equal width, vocabulary and number of layers)."""
+    layer_shapes_scenario(args, dev, "sagedra", "Sagedra", config_sagedra(), ("gumodra", config_gumodra()))
 
 
 def layer_shapes_scenario(args, dev, first, title, first_raw, other):
@@ -565,6 +626,9 @@ def layer_shapes_scenario(args, dev, first, title, first_raw, other):
             step_bytes = lambda b: gumodra_step_bytes(raw, esize, b, args.context)[0]
             params = gumodra_step_bytes(raw, esize, args.batch, 0)[1]
             prefill_params = gumodra_prefill_params(raw)
+        elif name == "sagedra":
+            step_bytes = lambda b: sagedra_step_bytes(raw, esize, b, args.context)[0]
+            params = sagedra_step_bytes(raw, esize, 0, 0)[1]
         else:
             step_bytes = lambda b: weight_bytes_per_step(cfg, esize) + b * args.context * kv_bytes_per_token(cfg, esize)
             params = weight_bytes_per_step(cfg, esize) // esize
@@ -620,6 +684,9 @@ def other_scenarios(args, dev):
         return
     if args.scenario == "gumodra":
         gumodra_scenario(args, dev)
+        return
+    if args.scenario == "sagedra":
+        sagedra_scenario(args, dev)
         return
     import torch
     from cpmcu_amd import Engine, EngineOptions, StepEntry

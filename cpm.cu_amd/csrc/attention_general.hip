@@ -507,9 +507,10 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
     // (four wavefronts that merge through LDS need room there beside the Q fragments)
     const long merge_bytes = (4 * 16 * 2 + 4L * dtm * 4 * 64) * 4;
     const int nw = (vs || (n <= 256 && q_bytes + merge_bytes <= 64 * 1024)) ? 4 : 1;
-    // tiles that pack several tokens: only where a wavefront has a tile to itself and nothing is merged
+    // tiles that pack several tokens: only where nothing is merged at the end (a wavefront has a tile to itself, or
+    // the four of a workgroup split the features of one tile)
     const int rpt = G < 16 ? G : 16;
-    CPMCU_REQUIRE(!tiles || (n_tiles > 0 && nw == 1 && n_splits == 1 && tokens_per_tile >= 1 && tokens_per_tile * rpt <= 16),
+    CPMCU_REQUIRE(!tiles || (n_tiles > 0 && (nw == 1 || vs) && n_splits == 1 && tokens_per_tile >= 1 && tokens_per_tile * rpt <= 16),
                   "attention_general_mfma: tiles of %d tokens do not suit this step", tokens_per_tile);
     const int tpt = tiles ? tokens_per_tile : 1;
     const int units = tiles ? n_tiles : n;

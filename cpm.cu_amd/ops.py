@@ -1504,7 +1504,7 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
     With n_splits > 1 every token's visible keys are shared among n_splits workgroups and merged afterwards;
     part_o float32 [n, nh, n_splits, hdv] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
     tiles (int32 [T, 2] = first packed token, tokens; prompts of more than 256 tokens with fewer than 16 heads a
-    kv head and values up to 128 features): runs of at most tokens_per_tile consecutive tokens of one sequence,
+    kv head): runs of at most tokens_per_tile consecutive tokens of one sequence,
     which share a matrix-core tile (tokens_per_tile * heads a kv head <= 16)."""
     _need(q, "attention q", torch.bfloat16, (None, nh * hdk))
     n = q.shape[0]
@@ -1535,10 +1535,10 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
 
 def attention_general_tokens_per_tile(n_tokens: int, nh: int, nkv: int, pool_hdv: int) -> int:
     """Tokens that share a matrix-core tile in attention_general_mfma: prompts of more than 256 tokens whose
-    kv heads serve fewer than 16 query heads (and whose values a wavefront holds alone) fill the tile's 16
-    columns with the heads of several consecutive tokens; 1 everywhere else."""
+    kv heads serve fewer than 16 query heads fill the tile's 16 columns with the heads of several consecutive
+    tokens; 1 everywhere else."""
     group = nh // nkv
-    if n_tokens <= 256 or pool_hdv > 128 or group > 8:
+    if n_tokens <= 256 or group > 8:
         return 1
     return 16 // group
 
