@@ -223,11 +223,15 @@ def test_rotation_then_unit_rms(dtype, shape):
 # ---------------------------------------------------------------------------
 # attention with two score maps a head
 
-def _diff_plain(q, k, v, scale, lam, eps, post, temp):
-    """q [T, H, 2, d], k [T, G, 2, d], v [T, G, dv]: the combined, normed heads [T, H*dv]."""
+def _diff_plain(q, k, v, scale, lam, eps, post, temp, q_dtype=None):
+    """q [T, H, 2, d], k [T, G, 2, d], v [T, G, dv]: the combined, normed heads [T, H*dv].  With q_dtype the
+    tempered queries are rounded to it, as the kernel stores them: where the temperature makes the softmax sharp,
+    that rounding alone moves the weights by more than every later step together."""
     T, H = q.shape[:2]
     rep = H // k.shape[1]
     q = q.double() * temp[:, None, None, None]
+    if q_dtype is not None:
+        q = q.to(q_dtype).double()
     k, v = k.double().repeat_interleave(rep, 1), v.double().repeat_interleave(rep, 1)
     mask = plain.visible(T)
     a1 = plain.softmax_attention(q[:, :, 0], k[:, :, 0], v, scale, mask)
@@ -308,10 +312,10 @@ def test_two_score_maps_over_shared_values(dtype, shape):
     torch.manual_seed(35)
     T, page, eps, coef, scale = 330, 64, 1e-5, 0.5, 0.3
     lam = math.exp(0.11) - math.exp(-0.2) + diff
-    src = torch.randn(T, 2 * H * d + 2 * G * d + G * dv)
+    src = torch.randn(T, 2 * H * d + 2 * G * d + G * dv).to(DT[dtype]).float()    # numbers that the type holds exactly
     q, k, v = src.split([2 * H * d, 2 * G * d, G * dv], 1)
     want, amp = _diff_plain(q.reshape(T, H, 2, d), k.reshape(T, G, 2, d), v.reshape(T, G, dv), scale, lam, eps, 1.0 - diff,
-                            _temperature(T, coef, every))
+                            _temperature(T, coef, every), DT[dtype] if dtype == "bfloat16" else None)
     checks = None
     if dtype == "bfloat16" and d % 8 == 0:
         checks = [(0, T, 1, False), (T - 40, T, 1, False), (T - 1, T, 5, False), (200, 201, 2, False), (T - 3, T, 1, False)]
