@@ -372,13 +372,15 @@ def _delta_plain(qkv, a, b, A_log, dt_bias, H, G, d, dv):
     return torch.stack([plain.delta_rule(q[:, i // rep], k[:, i // rep], v[:, i], beta[:, i], g[:, i]) for i in range(H)], 1).reshape(T, H * dv)
 
 
+@pytest.mark.parametrize("lanes", [0, 8, 16])
 @pytest.mark.parametrize("gates_dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape", [(4, 2, 24, 20), (1, 1, 72, 8), (2, 1, 12, 7), (3, 3, 8, 36), (4, 1, 32, 40), (4, 2, 128, 128),
-                                   (2, 2, 256, 16)])
-def test_delta_rule_in_portions_and_slots(gates_dtype, shape):
+                                   (2, 2, 256, 16), (2, 1, 200, 50)])
+def test_delta_rule_in_portions_and_slots(gates_dtype, shape, lanes):
     """Two sequences in slots 3 and 1, in portions of unequal sizes down to one token: the state is carried in the
     slot; a slot that is freed (its state cleared) and used again starts from nothing; a pass that does not write
-    leaves the state as it was.  Decays from nearly 1 to nearly 0, steps from nearly 0 to nearly 1."""
+    leaves the state as it was.  Decays from nearly 1 to nearly 0, steps from nearly 0 to nearly 1.  A column of
+    the state over 8 and over 16 lanes, and as the kernel chooses by the batch."""
     from cpmcu_amd import ops
     H, G, d, dv = shape
     torch.manual_seed(37)
@@ -405,7 +407,7 @@ def test_delta_rule_in_portions_and_slots(gates_dtype, shape):
         gates = dev(torch.cat([data[s][1][a:b] for s, a, b in batch]))
         y = torch.empty(cu[-1], H * dv, device=DEV)
         ops.delta_scan(qkv, gates, 3, 3 + H, dev(dt_bias), dev(A_log), state, y, i32(cu), i32([s for s, _, _ in batch]),
-                       H, G, d, dv, d ** -0.5, write_state=write)
+                       H, G, d, dv, d ** -0.5, write_state=write, lanes=lanes)
         return [y[cu[i]:cu[i + 1]].cpu() for i in range(len(batch))]
 
     for step in range(5):
