@@ -39,7 +39,7 @@ MODULES: Dict[str, List[str]] = {
 }
 HEADERS = ["common.h"]
 # headers of single libraries
-MODULE_HEADERS: Dict[str, List[str]] = {"attention": ["no_alloc.h"], "core": ["vec4.h"], "norms": ["vec4.h"]}
+MODULE_HEADERS: Dict[str, List[str]] = {"attention": ["no_alloc.h"], "core": ["vec4.h"], "norms": ["vec4.h"], "ssm": ["vec4.h"]}
 
 # -packed-fp32-ops off: the compiler must not form packed float instructions on its own
 HIPCC_FLAGS = [

@@ -8,21 +8,21 @@
 // Since S^T qn after the write is g (S_old^T qn) + (kn . qn) u, both products with the old state are formed in
 // one pass over it (a column's two sums meet in one reduction) and the state is read and written once a token.
 //
-// A workgroup owns one (sequence, head, 32 columns of dv) and walks the sequence's tokens in order; a column's
-// dk state values are spread over 8 neighbouring lanes (state index i = l + 8 r), the tokens' q, k, v and gates
-// pass through LDS in tiles of 16 or 32 tokens, where the unit norms and k . q are formed once a token, and the
-// next tile's values are asked for while the current one is walked.
+// A workgroup owns one (sequence, head, 32 or 16 columns of dv) and walks the sequence's tokens in order; a
+// column's dk state values are spread over 8 or 16 neighbouring lanes (state index i = l + L r), the tokens' q,
+// k, v and gates pass through LDS in tiles of 16 or 32 tokens, where the unit norms and k . q are formed once a
+// token, and the next tile's values are asked for while the current one is walked.  A token's cost is one
+// dependent chain of multiply-adds over a lane's share of the column and a reduction over the column's lanes:
+// where the batch has too few (sequence, head, column) triples to fill the chip (a single prompt, a step of one
+// sequence), 16 lanes a column halve that chain and double the number of workgroups.
 #include "common.h"
-
-#define DELTA_PB 32      // columns of dv a workgroup
-#define DELTA_L 8        // lanes a column
 
 __device__ inline float delta_softplus(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
 // qkv: float [n, ld] = [q: kv_heads*dk | k: kv_heads*dk | v: heads*dv] (after convolution and activation);
 // gates: raw projections [n, ldg], the decay's at column a_off + h, beta's at b_off + h;
 // state: float [slots][heads][dv][dk]; y: float [n, heads*dv].
-template <int NR, int TT, typename GT>
+template <int NR, int TT, int DELTA_L, typename GT>
 __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict__ qkv, long ld,
                                                          const GT* __restrict__ gates, long ldg, long a_off, long b_off,
                                                          const float* __restrict__ dt_bias,
@@ -30,6 +30,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
                                                          float* __restrict__ y, const int* __restrict__ cu_q,
                                                          const int* __restrict__ seq_slot, int heads, int kv_heads,
                                                          int dk, int dv, float q_scale, int write_state) {
+    constexpr int DELTA_PB = 256 / DELTA_L;         // columns of dv a workgroup
     constexpr int NS = NR * DELTA_L;                // state values a column, padded
     constexpr int QK = TT * NS / 256;               // q (and k) values a thread brings a tile
     constexpr int VV = (TT * DELTA_PB + 255) / 256; // v values a thread brings a tile
@@ -132,13 +133,17 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
                 r += S[i] * kr[i];
                 o += S[i] * qs[tt][n];
             }
-            // the column's 8 lanes are neighbours: both sums meet inside the vector unit, every lane gets them
+            // the column's lanes are neighbours: both sums meet inside the vector unit, every lane gets them
             r += CPMCU_DPP(r, 0xB1);
             o += CPMCU_DPP(o, 0xB1);
             r += CPMCU_DPP(r, 0x4E);
             o += CPMCU_DPP(o, 0x4E);
             r += CPMCU_DPP(r, 0x141);
             o += CPMCU_DPP(o, 0x141);
+            if (DELTA_L == 16) {
+                r += CPMCU_DPP(r, 0x140);
+                o += CPMCU_DPP(o, 0x140);
+            }
             const float u = beta * (vv - g * r);
 #pragma unroll
             for (int i = 0; i < NR; ++i) S[i] = g * S[i] + kr[i] * u;
@@ -157,28 +162,39 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
 extern "C" const char* cpmcu_delta_scan(const float* qkv, long ld, const void* gates, long ldg, int gate_dtype,
                                         long a_off, long b_off, const float* dt_bias, const float* A_log, float* state,
                                         float* y, const int* cu_q, const int* seq_slot, int n_seqs, int heads,
-                                        int kv_heads, int dk, int dv, float q_scale, int write_state,
+                                        int kv_heads, int dk, int dv, float q_scale, int write_state, int lanes,
                                         hipStream_t stream) {
     CPMCU_REQUIRE(n_seqs > 0 && heads > 0 && kv_heads > 0 && dk > 0 && dv > 0, "delta_scan: empty shape");
     CPMCU_REQUIRE(heads % kv_heads == 0, "delta_scan: %d heads are not a multiple of %d key heads", heads, kv_heads);
     CPMCU_REQUIRE(dk <= 256, "delta_scan: a key size of %d is not supported (at most 256)", dk);
     CPMCU_REQUIRE(ld >= 2L * kv_heads * dk + (long)heads * dv, "delta_scan: rows of %ld too short", ld);
     CPMCU_REQUIRE(a_off >= 0 && b_off >= 0 && ldg >= a_off + heads && ldg >= b_off + heads, "delta_scan: gate rows too short");
-    const int pb = (dv + DELTA_PB - 1) / DELTA_PB;
+    CPMCU_REQUIRE(lanes == 0 || lanes == 8 || lanes == 16, "delta_scan: %d lanes a column (0: chosen here, 8 or 16)", lanes);
+    // 16 lanes a column where 8 would leave fewer than two workgroups a compute unit and a column is long enough
+    if (lanes == 0) lanes = ((long)n_seqs * heads * ((dv + 31) / 32) < 512 && dk > 16 && dv > 16) ? 16 : 8;
+    const int cols = 256 / lanes;
+    const int pb = (dv + cols - 1) / cols;
     CPMCU_REQUIRE(heads <= 65535 && pb <= 65535, "delta_scan: shape exceeds the launch grid");
     dim3 grid(n_seqs, heads, pb);
-    const int need = (dk + DELTA_L - 1) / DELTA_L;
-#define LAUNCH(NRv, TTv, GTv)                                                                                       \
-    delta_scan_kernel<NRv, TTv, GTv><<<grid, 256, 0, stream>>>(qkv, ld, (const GTv*)gates, ldg, a_off, b_off, dt_bias, \
-                                                               A_log, state, y, cu_q, seq_slot, heads, kv_heads, dk,  \
-                                                               dv, q_scale, write_state)
-#define BY_NR(GTv)                                \
-    do {                                          \
-        if (need <= 2) LAUNCH(2, 32, GTv);        \
-        else if (need <= 4) LAUNCH(4, 32, GTv);   \
-        else if (need <= 8) LAUNCH(8, 32, GTv);   \
-        else if (need <= 16) LAUNCH(16, 32, GTv); \
-        else LAUNCH(32, 16, GTv);                 \
+    const int need = (dk + lanes - 1) / lanes;
+#define LAUNCH(NRv, TTv, Lv, GTv)                                                                                   \
+    delta_scan_kernel<NRv, TTv, Lv, GTv><<<grid, 256, 0, stream>>>(qkv, ld, (const GTv*)gates, ldg, a_off, b_off,     \
+                                                                   dt_bias, A_log, state, y, cu_q, seq_slot, heads,  \
+                                                                   kv_heads, dk, dv, q_scale, write_state)
+#define BY_NR(GTv)                                        \
+    do {                                                  \
+        if (lanes == 16) {                                \
+            if (need <= 2) LAUNCH(2, 32, 16, GTv);        \
+            else if (need <= 4) LAUNCH(4, 32, 16, GTv);   \
+            else if (need <= 8) LAUNCH(8, 32, 16, GTv);   \
+            else LAUNCH(16, 16, 16, GTv);                 \
+        } else {                                          \
+            if (need <= 2) LAUNCH(2, 32, 8, GTv);         \
+            else if (need <= 4) LAUNCH(4, 32, 8, GTv);    \
+            else if (need <= 8) LAUNCH(8, 32, 8, GTv);    \
+            else if (need <= 16) LAUNCH(16, 32, 8, GTv);  \
+            else LAUNCH(32, 16, 8, GTv);                  \
+        }                                                 \
     } while (0)
     if (gate_dtype == CPMCU_F32) BY_NR(float);
     else if (gate_dtype == CPMCU_BF16) BY_NR(bf16_t);

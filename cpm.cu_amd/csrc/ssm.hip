@@ -4,7 +4,8 @@
 //    column is the current token's; inputs before the sequence's start are zero) followed by SiLU, or by nothing.
 //    The sequence's last taps-1 inputs live in the slot's state, so a step continues where the last one ended.
 //    With in_bias the convolution's inputs are u + in_bias (a projection's bias that is still to be added); the
-//    state holds them with it, and the inputs before the start stay zero.
+//    state holds them with it, and the inputs before the start stay zero.  conv_silu_vec4_kernel is the same
+//    for 2 to 5 taps and channel counts that are multiples of 4: 4 channels a thread, the last inputs in registers.
 //  * conv_state_kernel: moves the step's last inputs into that state (after the convolution has read it); for
 //    steps of at most 16 tokens a sequence the convolution's kernel does that itself.
 //  * ssm_scan_kernel: the recurrence, per head h (group g = h / (heads / groups)):
@@ -17,6 +18,7 @@
 // column's N state values are spread over 8 neighbouring lanes, and the tokens' B, C, x and dt pass through
 // LDS in tiles of 16 or 32 tokens, the next tile asked for while the current one is worked on.
 #include "common.h"
+#include "vec4.h"
 
 __device__ inline float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
@@ -58,6 +60,88 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u
     }
 }
 
+// The same for channel counts and row strides that are multiples of 4: a thread owns 4 neighbouring channels
+// (8- or 16-byte loads, 16-byte stores) and walks its tile's tokens with the last TAPS-1 inputs in registers, so
+// every input is loaded once a tile instead of once a tap.  grid (sequences, token tiles, blocks of 1,024 channels).
+template <typename UT, int TAPS>
+__global__ __launch_bounds__(256) void conv_silu_vec4_kernel(const UT* __restrict__ u, long ldu,
+                                                             const float* __restrict__ weight,
+                                                             const float* __restrict__ bias,
+                                                             const float* state, float* __restrict__ out,
+                                                             const int* __restrict__ cu_q, const int* __restrict__ seq_slot,
+                                                             int C, int tile, float* state_out,
+                                                             const float* __restrict__ in_bias, int plain) {
+    const int b = blockIdx.x;
+    const int start = cu_q[b], q = cu_q[b + 1] - start;
+    const int slot = seq_slot[b];
+    const int c = (blockIdx.z * 256 + threadIdx.x) * 4;
+    if (c >= C) return;
+    const int i0 = blockIdx.y * tile, i1 = min(i0 + tile, q);
+    float w[4][TAPS];
+    {
+        float flat[4 * TAPS];
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
+            const float4 t = load4(weight + (long)c * TAPS + 4 * j);
+            flat[4 * j] = t.x; flat[4 * j + 1] = t.y; flat[4 * j + 2] = t.z; flat[4 * j + 3] = t.w;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int k = 0; k < TAPS; ++k) w[r][k] = flat[r * TAPS + k];
+    }
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4 bs = bias ? load4(bias + c) : zero;
+    const float4 ib = in_bias ? load4(in_bias + c) : zero;
+    const float* st = state + (long)slot * (TAPS - 1) * C + c;        // [slot][TAPS-1][C]
+    auto input = [&](int j) {                                          // the input at local index j >= 0
+        float4 t = load4(u + (long)(start + j) * ldu + c);
+        t.x += ib.x; t.y += ib.y; t.z += ib.z; t.w += ib.w;
+        return t;
+    };
+    float4 win[TAPS > 1 ? TAPS - 1 : 1];
+    if (i0 < i1) {
+#pragma unroll
+        for (int k = 0; k < TAPS - 1; ++k) {
+            const int j = i0 - (TAPS - 1) + k;
+            win[k] = j >= 0 ? input(j) : load4(st + (long)(TAPS - 1 + j) * C);
+        }
+    }
+    for (int i = i0; i < i1; i += 4) {
+        float4 cur[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cur[e] = input(min(i + e, i1 - 1));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (i + e < i1) {
+                float4 acc = bs;
+#pragma unroll
+                for (int k = 0; k < TAPS - 1; ++k) {
+                    acc.x += w[0][k] * win[k].x; acc.y += w[1][k] * win[k].y;
+                    acc.z += w[2][k] * win[k].z; acc.w += w[3][k] * win[k].w;
+                }
+                acc.x += w[0][TAPS - 1] * cur[e].x; acc.y += w[1][TAPS - 1] * cur[e].y;
+                acc.z += w[2][TAPS - 1] * cur[e].z; acc.w += w[3][TAPS - 1] * cur[e].w;
+                if (!plain) { acc.x = silu_f(acc.x); acc.y = silu_f(acc.y); acc.z = silu_f(acc.z); acc.w = silu_f(acc.w); }
+                store4(out + (long)(start + i + e) * C + c, acc.x, acc.y, acc.z, acc.w);
+#pragma unroll
+                for (int k = 0; k + 1 < TAPS - 1; ++k) win[k] = win[k + 1];
+                if (TAPS > 1) win[TAPS - 2] = cur[e];
+            }
+        }
+    }
+    // a step of one tile a sequence: this thread alone has read its channels' state and moves it on itself
+    if (state_out) {
+        float* so = state_out + (long)slot * (TAPS - 1) * C + c;
+#pragma unroll
+        for (int j = 0; j < TAPS - 1; ++j) {
+            const int i = q - (TAPS - 1) + j;
+            const float4 t = i >= 0 ? input(i) : load4(so + (long)(j + q) * C);
+            store4(so + (long)j * C, t.x, t.y, t.z, t.w);
+        }
+    }
+}
+
 // grid (sequences, channel blocks): state[j] <- the input at local index q - (taps-1) + j, which is one of the
 // step's tokens or, for a short step, an older entry of the state (read before it is overwritten: a thread
 // walks j upwards and reads index j + q > j).
@@ -92,7 +176,38 @@ extern "C" const char* cpmcu_conv_silu(const void* u, long ldu, int u_dtype, con
     dim3 grid(n_seqs, tb, cb), grid2(n_seqs, cb);
     const bool moves = update_state && taps > 1;
     float* fused = (moves && tb == 1) ? state : nullptr;
-    if (u_dtype == CPMCU_F32) {
+    const size_t esize = u_dtype == CPMCU_F32 ? 4 : 2;
+    const bool vec4 = taps >= 2 && taps <= 5 && C % 4 == 0 && ldu % 4 == 0 && (uintptr_t)u % (4 * esize) == 0 &&
+                      (uintptr_t)out % 16 == 0 && (uintptr_t)state % 16 == 0 && (uintptr_t)weight % 16 == 0 &&
+                      (!bias || (uintptr_t)bias % 16 == 0) && (!in_bias || (uintptr_t)in_bias % 16 == 0) &&
+                      (u_dtype == CPMCU_F32 || u_dtype == CPMCU_BF16);
+    if (vec4) {
+        // tiles of 16 tokens, of 64 where that still leaves the chip several workgroups a compute unit
+        const int cb4 = (C + 1023) / 1024;
+        const int tile = (tb > 1 && (long)n_seqs * ((max_q + 63) / 64) * cb4 >= 1024) ? 64 : 16;
+        dim3 grid4(n_seqs, (max_q + tile - 1) / tile, cb4);
+#define CONV4(UTv, TAPSv)                                                                                               \
+    conv_silu_vec4_kernel<UTv, TAPSv><<<grid4, 256, 0, stream>>>((const UTv*)u, ldu, weight, bias, state, out, cu_q,    \
+                                                                 seq_slot, C, tile, fused, in_bias, plain)
+#define CONV4_TAPS(UTv)                    \
+    do {                                   \
+        if (taps == 2) CONV4(UTv, 2);      \
+        else if (taps == 3) CONV4(UTv, 3); \
+        else if (taps == 4) CONV4(UTv, 4); \
+        else CONV4(UTv, 5);                \
+    } while (0)
+        if (u_dtype == CPMCU_F32) {
+            CONV4_TAPS(float);
+            if (moves && !fused)
+                conv_state_kernel<float><<<grid2, 256, 0, stream>>>((const float*)u, ldu, state, cu_q, seq_slot, C, taps, in_bias);
+        } else {
+            CONV4_TAPS(bf16_t);
+            if (moves && !fused)
+                conv_state_kernel<bf16_t><<<grid2, 256, 0, stream>>>((const bf16_t*)u, ldu, state, cu_q, seq_slot, C, taps, in_bias);
+        }
+#undef CONV4_TAPS
+#undef CONV4
+    } else if (u_dtype == CPMCU_F32) {
         conv_silu_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps, fused, in_bias, plain);
         if (moves && !fused)
             conv_state_kernel<float><<<grid2, 256, 0, stream>>>((const float*)u, ldu, state, cu_q, seq_slot, C, taps, in_bias);

@@ -882,13 +882,14 @@ def softcap(logits: torch.Tensor, cap: float):
 
 def delta_scan(qkv: torch.Tensor, gates: torch.Tensor, a_off: int, b_off: int, dt_bias: torch.Tensor,
                A_log: torch.Tensor, state: torch.Tensor, y: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor,
-               heads: int, kv_heads: int, dk: int, dv: int, q_scale: float, write_state: bool = True):
+               heads: int, kv_heads: int, dk: int, dv: int, q_scale: float, write_state: bool = True, lanes: int = 0):
     """The gated delta rule over each sequence's tokens, in float.  qkv float32 [n, 2*kv_heads*dk + heads*dv] =
     [q | k | v]; gates [n, W] holds the raw decay projection at columns a_off.. and the raw beta projection at
     b_off.. (heads each).  Per head (its q, k from head h // (heads/kv_heads)): q, k made unit vectors
     (x / sqrt(sum x^2 + 1e-6)), q times q_scale; beta = sigmoid(b); g = exp(-exp(A_log) softplus(a + dt_bias));
     S <- g S; u = beta (v - S^T k); S <- S + k u^T; y = S^T q.  state float32 [slots, heads, dv, dk]; y float32
-    [n, heads*dv]."""
+    [n, heads*dv].  lanes: how many lanes share a column of the state (8 or 16; 0: chosen by how much the batch
+    gives the chip to do)."""
     _need(qkv, "delta inputs", torch.float32, (None, 2 * kv_heads * dk + heads * dv))
     n = qkv.shape[0]
     ldg = _ld(gates, "delta gates")
@@ -904,7 +905,8 @@ def delta_scan(qkv: torch.Tensor, gates: torch.Tensor, a_off: int, b_off: int, d
     _check(_fn("delta", "cpmcu_delta_scan")(_p(qkv), c_long(qkv.shape[1]), _p(gates), c_long(ldg), c_int(_code(gates)),
                                             c_long(a_off), c_long(b_off), _p(dt_bias), _p(A_log), _p(state), _p(y),
                                             _p(cu_q), _p(seq_slot), c_int(B), c_int(heads), c_int(kv_heads), c_int(dk),
-                                            c_int(dv), c_float(q_scale), c_int(1 if write_state else 0), _stream()))
+                                            c_int(dv), c_float(q_scale), c_int(1 if write_state else 0), c_int(lanes),
+                                            _stream()))
 
 
 def diff_qkv_store(src: torch.Tensor, q_out: torch.Tensor, heads: int, kv_heads: int, dk: int, dv: int,
