@@ -92,14 +92,13 @@ __global__ __launch_bounds__(1024) void streams_norm_vec4_kernel(float* __restri
                                                                  const float* __restrict__ weight, float eps,
                                                                  OT* __restrict__ out, const int* __restrict__ rows, int H) {
     __shared__ float red[17];
-    __shared__ float mix_s[SM * SM], out_s[SM], read_s[SM];
     const long r = rows ? rows[blockIdx.x] : blockIdx.x;
-    if (threadIdx.x < S * S) mix_s[threadIdx.x] = mix ? mix[threadIdx.x] : ((threadIdx.x / S == threadIdx.x % S) ? 1.f : 0.f);
-    if (threadIdx.x < S) {
-        out_s[threadIdx.x] = outw ? outw[threadIdx.x] : 1.f;
-        read_s[threadIdx.x] = read ? read[threadIdx.x] : 1.f;
-    }
-    __syncthreads();
+    // the streams' numbers are the same for every thread: read where they are used, they come through the scalar
+    // unit beside the row's loads (staged through LDS, a barrier would stand between their arrival and the first
+    // load of the row)
+    auto mix_at = [&](int s_, int t_) { return mix ? mix[s_ * S + t_] : (s_ == t_ ? 1.f : 0.f); };
+    auto out_at = [&](int t_) { return outw ? outw[t_] : 1.f; };
+    auto read_at = [&](int t_) { return read ? read[t_] : 1.f; };
     const int H4 = H / 4;
     float4 u[4];
     float sum = 0.f;
@@ -120,16 +119,16 @@ __global__ __launch_bounds__(1024) void streams_norm_vec4_kernel(float* __restri
 #pragma unroll
             for (int t = 0; t < SM; ++t) {
                 if (t < S) {
-                    const float o = out_s[t];
+                    const float o = out_at(t);
                     float4 v = make_float4(o * y.x, o * y.y, o * y.z, o * y.w);
 #pragma unroll
                     for (int s = 0; s < SM; ++s)
                         if (s < S) {
-                            const float m = mix_s[s * S + t];
+                            const float m = mix_at(s, t);
                             v.x += m * xs[s].x; v.y += m * xs[s].y; v.z += m * xs[s].z; v.w += m * xs[s].w;
                         }
                     if (!rows) *(float4*)(xc + (long)t * stream_stride) = v;
-                    const float rd = read_s[t];
+                    const float rd = read_at(t);
                     a.x += rd * v.x; a.y += rd * v.y; a.z += rd * v.z; a.w += rd * v.w;
                 }
             }
@@ -137,7 +136,7 @@ __global__ __launch_bounds__(1024) void streams_norm_vec4_kernel(float* __restri
 #pragma unroll
             for (int t = 0; t < SM; ++t)
                 if (t < S) {
-                    const float rd = read_s[t];
+                    const float rd = read_at(t);
                     a.x += rd * xs[t].x; a.y += rd * xs[t].y; a.z += rd * xs[t].z; a.w += rd * xs[t].w;
                 }
         }
