@@ -490,7 +490,7 @@ def config_sagedra():
     temperature; pairs of a sliding-window attention (32 heads on 8 kv heads of 128, all features rotated with
     stretched frequencies, a window of 2,048, an output gate) beside a gated delta rule (32 heads on 16 key heads,
     128 by 128, 4 taps); GELU-gated feed-forwards of 11,008; a logit cap."""
-    diff = {"heads": 16, "kv_heads": 4, "dim": 128, "vdim": 256, "scale": 128 ** -0.5, "diff": 0.5, "conv": 4,
+    diff = {"heads": 16, "kv_heads": 4, "dim": 128, "vdim": 256, "scale": 128 ** -0.5, "diff": 0.35, "conv": 4,
             "q_temp": {"coef": 0.1, "every": 1024}}
     pair = {"left": {"heads": 32, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 1.0,
                      "rot": {"base": 500000.0, "dims": 128,
@@ -499,8 +499,8 @@ def config_sagedra():
             "right": {"heads": 32, "kv_heads": 16, "dim": 128, "vdim": 128, "conv": 4}}
     dense = {"kind": "dense", "ff": 11008}
     return {
-        "architecture": "Sagedra", "vocab": 73448, "width": 4096, "norm": {"eps": 1e-5}, "embedding": {"scale": 12.0},
-        "streams": 4, "logit_softcap": 30.0,
+        "architecture": "Sagedra", "vocab": 73448, "width": 4096, "norm": {"eps": 1e-6}, "embedding": {"scale": 64.0},
+        "streams": 4, "logit_softcap": 50.0,
         "layers": [
             {"type": "attention", "mixer": dict(diff), "mlp": dense},
             {"type": "parallel", "mixer": dict(pair), "mlp": dense},
