@@ -226,8 +226,8 @@ typedef float gfloatx4_t __attribute__((ext_vector_type(4)));
 // output row in one wavefront's registers.  Every key and value is loaded once, and nothing is merged at the end.
 template <int DTM, int NW, int TW, bool VS>
 __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
-    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o, float2* __restrict__ part_ml,
-    const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
+    const bf16_t* __restrict__ q, void* __restrict__ out, int out_f32, float* __restrict__ part_o,
+    float2* __restrict__ part_ml, const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk, int hdv,
     int pool_hdk, int pool_hdv, float scale_log2e, int chunk, int window, int keep_first, const float* __restrict__ sink,
     int n_splits, int n_tokens, const int* __restrict__ tiles, int n_tiles, int tpt, int rpt, int v_share) {
@@ -417,13 +417,19 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     if (n_splits == 1) {
         if (sink) l += exp2f(sink[head] * 1.4426950408889634f - m);
         const float inv = 1.0f / l;
-        bf16_t* o = out + ((long)t * nh + head) * hdv;
+        // the output as bf16, or as float for a consumer that goes on in float (a difference of two maps)
+        const long o0 = ((long)t * nh + head) * hdv;
 #pragma unroll
         for (int dt = 0; dt < DTM; ++dt) {
             if (dt0 + dt >= dtn || (NW > 1 && !VS && dt % NW != wave)) continue;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if ((dt0 + dt) * 16 + 4 * g + i < hdv) o[(dt0 + dt) * 16 + 4 * g + i] = f32_to_bf16(acc[dt][i] * inv);
+            for (int i = 0; i < 4; ++i) {
+                const int d = (dt0 + dt) * 16 + 4 * g + i;
+                if (d < hdv) {
+                    if (out_f32) ((float*)out)[o0 + d] = acc[dt][i] * inv;
+                    else ((bf16_t*)out)[o0 + d] = f32_to_bf16(acc[dt][i] * inv);
+                }
+            }
         }
     } else {
         const long idx = ((long)t * nh + head) * n_splits + split;
@@ -442,7 +448,7 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
 // out[token][head][:] = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s over up to 64 shares (a share without keys
 // has l = 0): lane s holds share s's (max, sum), the common maximum and the denominator are wave reductions.
 __global__ void attention_general_merge_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
-                                               bf16_t* __restrict__ out, int hdv, int n_splits,
+                                               void* __restrict__ out, int out_f32, int hdv, int n_splits,
                                                const float* __restrict__ sink, int nh) {
     const long row = blockIdx.x;
     const float2* ml = part_ml + row * n_splits;
@@ -469,11 +475,12 @@ __global__ void attention_general_merge_kernel(const float* __restrict__ part_o,
         }
         for (; s < n_splits; ++s)
             a += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv), s)) * po[(long)s * hdv + d];
-        out[row * hdv + d] = f32_to_bf16(a * inv);
+        if (out_f32) ((float*)out)[row * hdv + d] = a * inv;
+        else ((bf16_t*)out)[row * hdv + d] = f32_to_bf16(a * inv);
     }
 }
 
-extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, float* part_o, float* part_ml, int n,
+extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, int out_f32, float* part_o, float* part_ml, int n,
                                                     int nh, int nkv, int hdk, int hdv, int pool_hdk, int pool_hdv,
                                                     float scale, int chunk, int window, int keep_first,
                                                     const float* sink, const void* kpool, const void* vtpool,
@@ -521,7 +528,7 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
     dim3 grid((units + tw - 1) / tw, nkv * HT, n_splits);
 #define LAUNCH(DTMv, NWv, TWv, VSv)                                                                              \
     attention_general_mfma_kernel<DTMv, NWv, TWv, VSv><<<grid, NWv * TWv * 64, lds, stream>>>(                   \
-        (const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
+        (const bf16_t*)q, out, out_f32, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
         positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, window, keep_first, sink, n_splits, n,    \
         tiles, n_tiles, tpt, rpt, v_share)
     if (vs) {
@@ -542,7 +549,7 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
     if (n_splits > 1) {
         const unsigned rows = (unsigned)((long)n * nh);
         attention_general_merge_kernel<<<rows, hdv > 128 ? 256 : (hdv > 64 ? 128 : 64), 0, stream>>>(
-            part_o, (const float2*)part_ml, (bf16_t*)out, hdv, n_splits, sink, nh);
+            part_o, (const float2*)part_ml, out, out_f32, hdv, n_splits, sink, nh);
         CPMCU_LAUNCH_CHECK("attention_general_merge");
     }
     return nullptr;

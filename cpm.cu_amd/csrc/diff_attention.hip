@@ -76,14 +76,14 @@ extern "C" const char* cpmcu_diff_qkv_store(const void* src, long ld, int src_dt
 }
 
 // grid (tokens, H), a wavefront a (token, head); a [n, 2H, dv] in the order (kv head, map, head of the group)
-template <typename T>
-__global__ __launch_bounds__(64) void diff_combine_kernel(const T* __restrict__ a, T* __restrict__ out, int H, int G,
+template <typename AT, typename T>
+__global__ __launch_bounds__(64) void diff_combine_kernel(const AT* __restrict__ a, T* __restrict__ out, int H, int G,
                                                           int dv, float lambda, float eps, float post) {
     const long t = blockIdx.x;
     const int h = blockIdx.y, lane = threadIdx.x;
     const int rep = H / G, g = h / rep, j = h % rep;
-    const T* a1 = a + (t * 2 * H + (long)(2 * g) * rep + j) * dv;
-    const T* a2 = a1 + (long)rep * dv;
+    const AT* a1 = a + (t * 2 * H + (long)(2 * g) * rep + j) * dv;
+    const AT* a2 = a1 + (long)rep * dv;
     float ss = 0.f;
     for (int i = lane; i < dv; i += 64) {
         const float o = to_f32(a1[i]) - lambda * to_f32(a2[i]);
@@ -94,16 +94,18 @@ __global__ __launch_bounds__(64) void diff_combine_kernel(const T* __restrict__ 
     for (int i = lane; i < dv; i += 64) d[i] = from_f32<T>((to_f32(a1[i]) - lambda * to_f32(a2[i])) * r);
 }
 
-extern "C" const char* cpmcu_diff_combine(const void* a, void* out, int dtype, int n, int H, int G, int dv,
+extern "C" const char* cpmcu_diff_combine(const void* a, int a_dtype, void* out, int dtype, int n, int H, int G, int dv,
                                           float lambda, float eps, float post, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && H > 0 && G > 0 && dv > 0 && H % G == 0 && H <= 65535, "diff_combine: bad shape heads=%d kv_heads=%d", H, G);
     dim3 grid(n, H);
-    if (dtype == CPMCU_F32)
-        diff_combine_kernel<float><<<grid, 64, 0, stream>>>((const float*)a, (float*)out, H, G, dv, lambda, eps, post);
-    else if (dtype == CPMCU_BF16)
-        diff_combine_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)a, (bf16_t*)out, H, G, dv, lambda, eps, post);
+    if (a_dtype == CPMCU_F32 && dtype == CPMCU_F32)
+        diff_combine_kernel<float, float><<<grid, 64, 0, stream>>>((const float*)a, (float*)out, H, G, dv, lambda, eps, post);
+    else if (a_dtype == CPMCU_F32 && dtype == CPMCU_BF16)
+        diff_combine_kernel<float, bf16_t><<<grid, 64, 0, stream>>>((const float*)a, (bf16_t*)out, H, G, dv, lambda, eps, post);
+    else if (a_dtype == CPMCU_BF16 && dtype == CPMCU_BF16)
+        diff_combine_kernel<bf16_t, bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)a, (bf16_t*)out, H, G, dv, lambda, eps, post);
     else
-        CPMCU_FAIL("diff_combine: unknown dtype %d", dtype);
+        CPMCU_FAIL("diff_combine: unsupported dtypes maps=%d out=%d", a_dtype, dtype);
     CPMCU_LAUNCH_CHECK("diff_combine");
     return nullptr;
 }

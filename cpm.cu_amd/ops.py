@@ -943,11 +943,11 @@ def diff_qkv_store(src: torch.Tensor, q_out: torch.Tensor, heads: int, kv_heads:
 def diff_combine(a: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, dv: int, lam: float, eps: float,
                  post: float):
     """out[t, h] = o / sqrt(mean(o^2) + eps) * post with o = a1 - lam * a2, the two maps' attention outputs of head
-    h; a [n, 2*heads*dv] in the order (kv head, map, head of the group), out [n, heads*dv]."""
+    h; a [n, 2*heads*dv] in the order (kv head, map, head of the group; float32, or out's type), out [n, heads*dv]."""
     _need(a, "diff maps", shape=(None, 2 * heads * dv))
     n = a.shape[0]
-    _need(out, "diff out", a.dtype, (n, heads * dv))
-    _check(_fn("attention_general", "cpmcu_diff_combine")(_p(a), _p(out), c_int(_code(a)), c_int(n), c_int(heads),
+    _need(out, "diff out", shape=(n, heads * dv))
+    _check(_fn("attention_general", "cpmcu_diff_combine")(_p(a), c_int(_code(a)), _p(out), c_int(_code(out)), c_int(n), c_int(heads),
                                                           c_int(kv_heads), c_int(dv), c_float(lam), c_float(eps),
                                                           c_float(post), _stream()))
 
@@ -1507,10 +1507,13 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
     part_o float32 [n, nh, n_splits, hdv] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
     tiles (int32 [T, 2] = first packed token, tokens; prompts of more than 256 tokens with fewer than 16 heads a
     kv head): runs of at most tokens_per_tile consecutive tokens of one sequence,
-    which share a matrix-core tile (tokens_per_tile * heads a kv head <= 16)."""
+    which share a matrix-core tile (tokens_per_tile * heads a kv head <= 16).  out is bfloat16, or float32 for a
+    consumer that goes on in float (a difference of two maps)."""
     _need(q, "attention q", torch.bfloat16, (None, nh * hdk))
     n = q.shape[0]
-    _need(out, "attention out", torch.bfloat16, (n, nh * hdv))
+    if out.dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError(f"attention out: dtype {out.dtype} (bfloat16 or float32)")
+    _need(out, "attention out", out.dtype, (n, nh * hdv))
     _need(kpool, "attention key pool", torch.bfloat16, (None, page_size, None))
     _need(vpool, "attention value pool", torch.bfloat16, (kpool.shape[0], page_size, None))
     nvh = _value_heads(nkv, v_share)
@@ -1527,7 +1530,8 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
     if sink is not None:
         _need(sink, "attention sink", torch.float32, (nh,))
     _check(_fn("attention_general", "cpmcu_attention_general_mfma")(
-        _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hdk), c_int(hdv),
+        _p(q), _p(out), c_int(1 if out.dtype == torch.float32 else 0), _p(part_o), _p(part_ml), c_int(n), c_int(nh),
+        c_int(nkv), c_int(hdk), c_int(hdv),
         c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nvh), c_float(scale), c_int(chunk), c_int(window),
         c_int(keep_first), _p(sink), _p(kpool), _p(vpool),
         _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot), c_int(n_splits),
@@ -1560,8 +1564,8 @@ def reserve_attention_general(ws, dtype, nh: int, nkv: int, hdv: int, pool_hdv: 
 def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx, chunk: int = 0,
                   window: int = 0, keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1):
     """Attention with key and value sizes of their own and an optional mask (chunks, or a sliding window with kept
-    first tokens) and softmax sink, with the kernel that suits the step; writes ``out`` [n, nh*hdv].  v_share:
-    runs of that many neighbouring key heads read one value head."""
+    first tokens) and softmax sink, with the kernel that suits the step; writes ``out`` [n, nh*hdv] (q's type, or
+    float32).  v_share: runs of that many neighbouring key heads read one value head."""
     pool_hdv = vpool.shape[2] // _value_heads(nkv, v_share)
     if (hdk == hdv and chunk == 0 and window == 0 and sink is None and hdk <= 256 and hdk % 16 == 0
             and kpool.shape[2] == nkv * hdk and v_share == 1):
@@ -1589,6 +1593,13 @@ def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, pa
                     tiles = ctx.extras[key] = prefill_tiles(ctx.q_lens, tpt, q.device)
         attention_general_mfma(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
                                ctx.tok_slot, chunk, splits, part_o, part_ml, tiles, tpt, window, keep_first, sink, v_share)
+        return
+    if out.dtype != q.dtype:
+        # the plain kernel writes the type it reads: through scratch of that type
+        tmp = ctx.ws.get("attn.gout_plain", tuple(out.shape), q.dtype)
+        attention_general(q, tmp, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
+                          ctx.tok_slot, chunk, window, keep_first, sink, v_share)
+        out.copy_(tmp)
         return
     attention_general(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
                       ctx.tok_slot, chunk, window, keep_first, sink, v_share)

@@ -102,7 +102,9 @@ class DifferentialAttention(Mixer):
             q = ctx.ws.get("dattn.q", (n, 2 * H * dk), self.rt.dtype)
             ops.diff_qkv_store(mixed, q, H, G, dk, dv, self.temp_coef, self.temp_every, ctx.positions, ctx.tok_slot,
                                cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size)
-        maps = ctx.ws.get("dattn.maps", (n, 2 * H * dv), self.rt.dtype)
+        # the two maps' outputs stay float: where they nearly cancel, their difference would carry bf16's rounding
+        # of each, enlarged by the division that follows
+        maps = ctx.ws.get("dattn.maps", (n, 2 * H * dv), torch.float32)
         with ctx.timed("attn_core"):
             ops.attention_any(q, maps, 2 * H, 2 * G, dk, dv, self.scale, cache.streams["k"], cache.streams["v"],
                               cache.page_table, cache.page_size, ctx, v_share=2)

@@ -283,8 +283,9 @@ def _diff_run(ops, src, H, G, d, dv, scale, lam, eps, post, coef, every, page, p
     out = torch.empty(T, H * dv, dtype=DT[dtype], device=DEV)
     ops.diff_combine(maps, out, H, G, dv, lam, eps, post)
     outs = [(0, T, out)]
-    for a, b, splits, tiled in (mfma_checks or []):
-        m2 = torch.empty(b - a, 2 * H * dv, dtype=torch.bfloat16, device=DEV)
+    for i, (a, b, splits, tiled) in enumerate(mfma_checks or []):
+        # the maps leave the matrix-core kernel (and the merge of split keys) as float, as the mixer asks, or as bf16
+        m2 = torch.empty(b - a, 2 * H * dv, dtype=torch.float32 if i != 1 else torch.bfloat16, device=DEV)
         po = torch.empty(b - a, 2 * H, splits, dv, device=DEV) if splits > 1 else None
         pm = torch.empty(b - a, 2 * H, splits, 2, device=DEV) if splits > 1 else None
         tiles, tpt = None, 1
