@@ -230,7 +230,8 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     float2* __restrict__ part_ml, const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk, int hdv,
     int pool_hdk, int pool_hdv, float scale_log2e, int chunk, int window, int keep_first, const float* __restrict__ sink,
-    int n_splits, int n_tokens, const int* __restrict__ tiles, int n_tiles, int tpt, int rpt, int v_share) {
+    int n_splits, int n_tokens, const int* __restrict__ tiles, int n_tiles, int tpt, int rpt, int v_share,
+    const bf16_t* __restrict__ gate, long ld_gate) {
     extern __shared__ __align__(16) unsigned char smem[];
     static_assert(NW == 1 || TW == 1, "either the wavefronts of a workgroup share a token or each has its own");
     const int ksteps = (pool_hdk + 31) >> 5, dtn = pool_hdv >> 4;
@@ -426,8 +427,11 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
             for (int i = 0; i < 4; ++i) {
                 const int d = (dt0 + dt) * 16 + 4 * g + i;
                 if (d < hdv) {
-                    if (out_f32) ((float*)out)[o0 + d] = acc[dt][i] * inv;
-                    else ((bf16_t*)out)[o0 + d] = f32_to_bf16(acc[dt][i] * inv);
+                    float v = acc[dt][i] * inv;
+                    // an output gate: times sigmoid of the token's gate row (heads side by side)
+                    if (gate) v /= 1.0f + expf(-to_f32(gate[(long)t * ld_gate + (long)head * hdv + d]));
+                    if (out_f32) ((float*)out)[o0 + d] = v;
+                    else ((bf16_t*)out)[o0 + d] = f32_to_bf16(v);
                 }
             }
         }
@@ -449,7 +453,8 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
 // has l = 0): lane s holds share s's (max, sum), the common maximum and the denominator are wave reductions.
 __global__ void attention_general_merge_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
                                                void* __restrict__ out, int out_f32, int hdv, int n_splits,
-                                               const float* __restrict__ sink, int nh) {
+                                               const float* __restrict__ sink, int nh,
+                                               const bf16_t* __restrict__ gate, long ld_gate) {
     const long row = blockIdx.x;
     const float2* ml = part_ml + row * n_splits;
     const float* po = part_o + row * n_splits * hdv;
@@ -475,8 +480,10 @@ __global__ void attention_general_merge_kernel(const float* __restrict__ part_o,
         }
         for (; s < n_splits; ++s)
             a += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv), s)) * po[(long)s * hdv + d];
-        if (out_f32) ((float*)out)[row * hdv + d] = a * inv;
-        else ((bf16_t*)out)[row * hdv + d] = f32_to_bf16(a * inv);
+        float r = a * inv;
+        if (gate) r /= 1.0f + expf(-to_f32(gate[(row / nh) * ld_gate + (row % nh) * hdv + d]));
+        if (out_f32) ((float*)out)[row * hdv + d] = r;
+        else ((bf16_t*)out)[row * hdv + d] = f32_to_bf16(r);
     }
 }
 
@@ -487,8 +494,9 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, in
                                                     const int* page_table, int table_width, int page_size,
                                                     const int* positions, const int* tok_slot, int n_splits,
                                                     const int* tiles, int n_tiles, int tokens_per_tile, int v_share,
-                                                    hipStream_t stream) {
+                                                    const void* gate, long ld_gate, hipStream_t stream) {
     CPMCU_REQUIRE(v_share >= 1 && nkv % v_share == 0, "attention_general_mfma: %d key heads do not share values in runs of %d", nkv, v_share);
+    CPMCU_REQUIRE(!gate || ld_gate >= (long)nh * hdv, "attention_general_mfma: gate rows of %ld elements for %d heads of %d", ld_gate, nh, hdv);
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_general_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
     CPMCU_REQUIRE(hdk > 0 && hdk % 8 == 0 && hdk <= 1024 && hdv > 0 && hdv <= 512,
                   "attention_general_mfma: key size %d (a multiple of 8 up to 1024) / value size %d (up to 512) have no "
@@ -530,7 +538,7 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, in
     attention_general_mfma_kernel<DTMv, NWv, TWv, VSv><<<grid, NWv * TWv * 64, lds, stream>>>(                   \
         (const bf16_t*)q, out, out_f32, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
         positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, window, keep_first, sink, n_splits, n,    \
-        tiles, n_tiles, tpt, rpt, v_share)
+        tiles, n_tiles, tpt, rpt, v_share, n_splits == 1 ? (const bf16_t*)gate : nullptr, ld_gate)
     if (vs) {
         if (dtm == 4) LAUNCH(4, 4, 1, true);
         else LAUNCH(8, 4, 1, true);
@@ -549,7 +557,7 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, in
     if (n_splits > 1) {
         const unsigned rows = (unsigned)((long)n * nh);
         attention_general_merge_kernel<<<rows, hdv > 128 ? 256 : (hdv > 64 ? 128 : 64), 0, stream>>>(
-            part_o, (const float2*)part_ml, out, out_f32, hdv, n_splits, sink, nh);
+            part_o, (const float2*)part_ml, out, out_f32, hdv, n_splits, sink, nh, (const bf16_t*)gate, ld_gate);
         CPMCU_LAUNCH_CHECK("attention_general_merge");
     }
     return nullptr;

@@ -1501,14 +1501,16 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
                            positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0, n_splits: int = 1,
                            part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                            tiles: Optional[torch.Tensor] = None, tokens_per_tile: int = 1, window: int = 0,
-                           keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1):
+                           keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1,
+                           gate: Optional[torch.Tensor] = None):
     """attention_general in bf16 on the matrix cores (key size a multiple of 8 up to 1024, value size up to 512).
     With n_splits > 1 every token's visible keys are shared among n_splits workgroups and merged afterwards;
     part_o float32 [n, nh, n_splits, hdv] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
     tiles (int32 [T, 2] = first packed token, tokens; prompts of more than 256 tokens with fewer than 16 heads a
     kv head): runs of at most tokens_per_tile consecutive tokens of one sequence,
     which share a matrix-core tile (tokens_per_tile * heads a kv head <= 16).  out is bfloat16, or float32 for a
-    consumer that goes on in float (a difference of two maps)."""
+    consumer that goes on in float (a difference of two maps).  gate (bfloat16 [n, nh*hdv], may be a column slice
+    of a wider projection): the output is multiplied element by element with sigmoid(gate) before it is written."""
     _need(q, "attention q", torch.bfloat16, (None, nh * hdk))
     n = q.shape[0]
     if out.dtype not in (torch.bfloat16, torch.float32):
@@ -1529,6 +1531,11 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
         _need(tiles, "attention tiles", torch.int32, (None, 2))
     if sink is not None:
         _need(sink, "attention sink", torch.float32, (nh,))
+    ld_gate = 0
+    if gate is not None:
+        ld_gate = _ld(gate, "attention gate")
+        if gate.dtype != torch.bfloat16 or tuple(gate.shape) != (n, nh * hdv):
+            raise KernelError(f"attention gate: {gate.dtype} {tuple(gate.shape)}, expected bfloat16 {(n, nh * hdv)}")
     _check(_fn("attention_general", "cpmcu_attention_general_mfma")(
         _p(q), _p(out), c_int(1 if out.dtype == torch.float32 else 0), _p(part_o), _p(part_ml), c_int(n), c_int(nh),
         c_int(nkv), c_int(hdk), c_int(hdv),
@@ -1536,7 +1543,7 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
         c_int(keep_first), _p(sink), _p(kpool), _p(vpool),
         _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot), c_int(n_splits),
         _p(tiles), c_int(tiles.shape[0] if tiles is not None else 0), c_int(tokens_per_tile), c_int(v_share),
-        _stream()))
+        _p(gate), c_long(ld_gate), _stream()))
 
 
 def attention_general_tokens_per_tile(n_tokens: int, nh: int, nkv: int, pool_hdv: int) -> int:
@@ -1562,15 +1569,18 @@ def reserve_attention_general(ws, dtype, nh: int, nkv: int, hdv: int, pool_hdv: 
 
 
 def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx, chunk: int = 0,
-                  window: int = 0, keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1):
+                  window: int = 0, keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1,
+                  gate: Optional[torch.Tensor] = None) -> bool:
     """Attention with key and value sizes of their own and an optional mask (chunks, or a sliding window with kept
     first tokens) and softmax sink, with the kernel that suits the step; writes ``out`` [n, nh*hdv] (q's type, or
-    float32).  v_share: runs of that many neighbouring key heads read one value head."""
+    float32).  v_share: runs of that many neighbouring key heads read one value head.  gate [n, nh*hdv]: an output
+    gate that the matrix-core kernel applies as it writes (out * sigmoid(gate)); returns whether it did, so that
+    the caller applies it itself after the other kernels."""
     pool_hdv = vpool.shape[2] // _value_heads(nkv, v_share)
     if (hdk == hdv and chunk == 0 and window == 0 and sink is None and hdk <= 256 and hdk % 16 == 0
             and kpool.shape[2] == nkv * hdk and v_share == 1):
         attention(q, out, nh, nkv, hdk, scale, kpool, vpool, page_table, page_size, ctx)
-        return
+        return False
     if attention_general_mfma_ok(q, hdk, hdv, page_size):
         n = q.shape[0]
         keys = ctx.max_pos + 1
@@ -1592,14 +1602,16 @@ def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, pa
                 if tiles is None:
                     tiles = ctx.extras[key] = prefill_tiles(ctx.q_lens, tpt, q.device)
         attention_general_mfma(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
-                               ctx.tok_slot, chunk, splits, part_o, part_ml, tiles, tpt, window, keep_first, sink, v_share)
-        return
+                               ctx.tok_slot, chunk, splits, part_o, part_ml, tiles, tpt, window, keep_first, sink, v_share,
+                               gate)
+        return gate is not None
     if out.dtype != q.dtype:
         # the plain kernel writes the type it reads: through scratch of that type
         tmp = ctx.ws.get("attn.gout_plain", tuple(out.shape), q.dtype)
         attention_general(q, tmp, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
                           ctx.tok_slot, chunk, window, keep_first, sink, v_share)
         out.copy_(tmp)
-        return
+        return False
     attention_general(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
                       ctx.tok_slot, chunk, window, keep_first, sink, v_share)
+    return False

@@ -338,14 +338,16 @@ class GeneralAttention(Mixer):
                                      cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
                                      write_kv=writes_cache)
         out = ctx.ws.get("attn.out", (n, nh * dv), self.rt.dtype)
+        gate = qkv[:, self.gate_off:self.gate_off + nh * dv] if self.gate_off is not None else None
         with ctx.timed("attn_core"):
-            ops.attention_any(q, out, nh, nkv, dk, dv, self.scale, cache.streams["k"], cache.streams["v"],
-                              cache.page_table, cache.page_size, ctx, chunk=self.chunk, window=self.window,
-                              keep_first=self.keep_first, sink=self.sink)
-        if self.gate_off is not None:
+            # the matrix-core kernel (and the merge of split keys) applies the gate as it writes
+            gated_there = ops.attention_any(q, out, nh, nkv, dk, dv, self.scale, cache.streams["k"], cache.streams["v"],
+                                            cache.page_table, cache.page_size, ctx, chunk=self.chunk, window=self.window,
+                                            keep_first=self.keep_first, sink=self.sink, gate=gate)
+        if gate is not None and not gated_there:
             with ctx.timed("attn_gate"):
                 gated = ctx.ws.get("attn.gated", (n, nh * dv), self.rt.dtype)
-                ops.sigmoid_gate(out, qkv[:, self.gate_off:self.gate_off + nh * dv], gated)
+                ops.sigmoid_gate(out, gate, gated)
                 out = gated
         with ctx.timed("attn_o"):
             branch = self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)

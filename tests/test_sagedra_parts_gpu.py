@@ -220,6 +220,51 @@ def test_rotation_then_unit_rms(dtype, shape):
     close(out[29:], want.reshape(T, H * dv)[29:], dtype)
 
 
+@pytest.mark.parametrize("shape", [(6, 2, 24, 40), (2, 2, 32, 16), (4, 1, 64, 64), (8, 8, 16, 24), (32, 8, 128, 128)])
+def test_output_gate_in_the_attention_kernel(shape):
+    """The matrix-core kernel multiplies what it writes with sigmoid of a gate row (a column slice of a wider
+    projection): prompts a token a tile and in token tiles, single tokens with whole and with split keys."""
+    from cpmcu_amd import ops
+    H, G, d, dv = shape
+    torch.manual_seed(39)
+    T, page, eps = 300, 64, 1e-5
+    row = torch.randn(T, H * d + G * d + G * dv).bfloat16()
+    pos = torch.arange(T)
+    q_raw, k_raw, v_raw = row.double().split([H * d, G * d, G * dv], 1)
+    k_want = plain.rms(k_raw.reshape(T, G, d), eps)
+    pk, pv = -(-d // 16) * 16, -(-dv // 16) * 16
+    kp = torch.zeros(6, page, G * pk, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros(6, page, G * pv, dtype=torch.bfloat16, device=DEV)
+    table = torch.zeros(2, 5, dtype=torch.int32)
+    table[1] = torch.tensor([3, 0, 4, 1, 5])
+    slot = i32([1] * T)
+    q_out = torch.empty(T, H * d, dtype=torch.bfloat16, device=DEV)
+    ops.qkv_norm_rotate_store(dev(row), q_out, H, G, d, dv, 0, i32(pos.tolist()), slot, None, 1.0, kp, vp, dev(table), page,
+                              eps=eps, norm_after=True)
+    qq = torch.randn(T, H, d).bfloat16()
+    wide = (torch.randn(T, H * dv + 9) * 2).bfloat16()                   # the gate's rows lie at column 4 of wider rows
+    gate = dev(wide)[:, 4:4 + H * dv]
+    want = plain.softmax_attention(qq.double(), k_want.repeat_interleave(H // G, 1),
+                                   v_raw.reshape(T, G, dv).repeat_interleave(H // G, 1), 0.4, plain.visible(T, 90))
+    want = want.reshape(T, H * dv) * torch.sigmoid(wide[:, 4:4 + H * dv].double())
+    q = dev(qq.reshape(T, H * d))
+    cases = [(0, T, 1, False), (T - 1, T, 1, False), (T - 1, T, 3, False), (150, 151, 2, False)]
+    if H // G <= 8:
+        cases.append((0, T, 1, True))
+    for a, b, splits, tiled in cases:
+        out = torch.empty(b - a, H * dv, dtype=torch.bfloat16, device=DEV)
+        po = torch.empty(b - a, H, splits, dv, device=DEV) if splits > 1 else None
+        pm = torch.empty(b - a, H, splits, 2, device=DEV) if splits > 1 else None
+        tiles, tpt = None, 1
+        if tiled:
+            tpt = ops.attention_general_tokens_per_tile(b - a, H, G, pv)
+            assert tpt > 1
+            tiles = ops.prefill_tiles([b - a], tpt, DEV)
+        ops.attention_general_mfma(q[a:b], out, H, G, d, dv, 0.4, kp, vp, dev(table), page, i32(pos[a:b].tolist()), slot[a:b],
+                                   0, splits, po, pm, tiles, tpt, window=90, gate=gate[a:b])
+        close(out, want[a:b], "bfloat16", what=f"rows {a}..{b} splits {splits} tiled {tiled}")
+
+
 # ---------------------------------------------------------------------------
 # attention with two score maps a head
 
