@@ -3,3 +3,4 @@ from .minicpm import MiniCPMConfig, RopeScaling, SparseConfig
 from .duvulix import DuvulixConfig
 from .gumodra import GumodraConfig
 from .sagedra import SagedraConfig
+from .nelutar import NelutarConfig

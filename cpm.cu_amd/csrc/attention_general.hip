@@ -104,7 +104,7 @@ __global__ __launch_bounds__(64) void attention_general_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ kpool, const T* __restrict__ vpool,
     PagedView pv, const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk,
     int hdv, int pool_hdk, int pool_hdv, float scale, int chunk, int window, int keep_first,
-    const float* __restrict__ sink, int v_share) {
+    const float* __restrict__ sink, int v_share, float softcap) {
     __shared__ float qs[AG_MAX_HD];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int g = h / (nh / nkv);
@@ -132,6 +132,7 @@ __global__ __launch_bounds__(64) void attention_general_kernel(
             float dot = 0.f;
             for (int d = 0; d < hdk; ++d) dot += qs[d] * to_f32(kr[key_d_offset(d)]);
             s = dot * scale;
+            if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         }
         const float m_new = fmaxf(m, wave_max(s));
         const float p = valid ? expf(s - m_new) : 0.f;
@@ -168,7 +169,7 @@ extern "C" const char* cpmcu_attention_general(const void* q, void* out, int dty
                                                const void* vpool,
                                                const int* page_table, int table_width, int page_size,
                                                const int* positions, const int* tok_slot, int v_share,
-                                               hipStream_t stream) {
+                                               float softcap, hipStream_t stream) {
     CPMCU_REQUIRE(v_share >= 1 && nkv % v_share == 0, "attention_general: %d key heads do not share values in runs of %d", nkv, v_share);
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && hdk > 0 && hdv > 0,
                   "attention_general: empty shape n=%d heads=%d kv_heads=%d key size=%d value size=%d", n, nh, nkv, hdk, hdv);
@@ -188,12 +189,12 @@ extern "C" const char* cpmcu_attention_general(const void* q, void* out, int dty
         attention_general_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, (float*)out, (const float*)kpool,
                                                                  (const float*)vpool, pv, positions, tok_slot, nh, nkv,
                                                                  hdk, hdv, pool_hdk, pool_hdv, scale, chunk, window,
-                                                                 keep_first, sink, v_share);
+                                                                 keep_first, sink, v_share, softcap);
     else if (dtype == CPMCU_BF16)
         attention_general_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kpool,
                                                                   (const bf16_t*)vpool, pv, positions, tok_slot, nh,
                                                                   nkv, hdk, hdv, pool_hdk, pool_hdv, scale, chunk, window,
-                                                                  keep_first, sink, v_share);
+                                                                  keep_first, sink, v_share, softcap);
     else
         CPMCU_FAIL("attention_general: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("attention_general");
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk, int hdv,
     int pool_hdk, int pool_hdv, float scale_log2e, int chunk, int window, int keep_first, const float* __restrict__ sink,
     int n_splits, int n_tokens, const int* __restrict__ tiles, int n_tiles, int tpt, int rpt, int v_share,
-    const bf16_t* __restrict__ gate, long ld_gate) {
+    const bf16_t* __restrict__ gate, long ld_gate, float cap_in, float cap_out) {
     extern __shared__ __align__(16) unsigned char smem[];
     static_assert(NW == 1 || TW == 1, "either the wavefronts of a workgroup share a token or each has its own");
     const int ksteps = (pool_hdk + 31) >> 5, dtn = pool_hdv >> 4;
@@ -337,6 +338,15 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
             }
         }
         // lane (head n, g): st0[e] is key key0 + 8g + e, st1[e] is key key0 + 8g + 4 + e
+        if (cap_out > 0.f) {
+            // capped scores c tanh(s scale / c), here already times log2(e): cap_in = scale / c, cap_out = c log2(e),
+            // and scale_log2e is 1 for the softmax below
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                st0[e] = cap_out * tanhf(st0[e] * cap_in);
+                st1[e] = cap_out * tanhf(st1[e] * cap_in);
+            }
+        }
         if (key0 + 31 > pos_min || (key0 < first_max && key0 + 31 >= keep_first)) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -494,7 +504,7 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, in
                                                     const int* page_table, int table_width, int page_size,
                                                     const int* positions, const int* tok_slot, int n_splits,
                                                     const int* tiles, int n_tiles, int tokens_per_tile, int v_share,
-                                                    const void* gate, long ld_gate, hipStream_t stream) {
+                                                    const void* gate, long ld_gate, float softcap, hipStream_t stream) {
     CPMCU_REQUIRE(v_share >= 1 && nkv % v_share == 0, "attention_general_mfma: %d key heads do not share values in runs of %d", nkv, v_share);
     CPMCU_REQUIRE(!gate || ld_gate >= (long)nh * hdv, "attention_general_mfma: gate rows of %ld elements for %d heads of %d", ld_gate, nh, hdv);
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_general_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
@@ -511,7 +521,8 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, in
     const int G = nh / nkv, HT = (G + 15) / 16;
     CPMCU_REQUIRE((long)nkv * HT <= 65535, "attention_general_mfma: too many head tiles");
     PagedView pv{page_table, table_width, page_size};
-    const float sl = scale * 1.4426950408889634f;
+    const float sl = softcap > 0.f ? 1.0f : scale * 1.4426950408889634f;
+    const float cap_in = softcap > 0.f ? scale / softcap : 0.f, cap_out = softcap > 0.f ? softcap * 1.4426950408889634f : 0.f;
     const int ksteps = (pool_hdk + 31) / 32, dtn = pool_hdv / 16;
     const long q_bytes = (long)ksteps * 64 * 16;
     // values up to 128 features: few tokens: 4 wavefronts share a token's keys and merge through LDS; many: a
@@ -538,7 +549,7 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, in
     attention_general_mfma_kernel<DTMv, NWv, TWv, VSv><<<grid, NWv * TWv * 64, lds, stream>>>(                   \
         (const bf16_t*)q, out, out_f32, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
         positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, window, keep_first, sink, n_splits, n,    \
-        tiles, n_tiles, tpt, rpt, v_share, n_splits == 1 ? (const bf16_t*)gate : nullptr, ld_gate)
+        tiles, n_tiles, tpt, rpt, v_share, n_splits == 1 ? (const bf16_t*)gate : nullptr, ld_gate, cap_in, cap_out)
     if (vs) {
         if (dtm == 4) LAUNCH(4, 4, 1, true);
         else LAUNCH(8, 4, 1, true);
@@ -568,18 +579,21 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, in
 // ===========================================================================
 template <typename IT, typename OT>
 __device__ inline void rotate_run(const IT* __restrict__ s, OT* __restrict__ d, int width, int rot_dims, int pos,
-                                  const float* __restrict__ inv_freq, float mag, int mode, int f0, int lane, int nl) {
+                                  const float* __restrict__ inv_freq, float mag, int mode, int f0, int lane, int nl,
+                                  int interleaved = 0) {
     auto at = [&](int i) -> long {
         if (mode == DST_ROWS) return i;
         return mode == DST_KEYS ? key_d_offset(f0 + i) : value_d_offset(f0 + i);
     };
+    // pair i of the rotation: features (i, i + rot_dims/2), or neighbours (2i, 2i + 1) when interleaved
     const int half = rot_dims / 2;
     for (int i = lane; i < half; i += nl) {
         const float ang = (float)pos * inv_freq[i];
         const float cs = cosf(ang) * mag, sn = sinf(ang) * mag;
-        const float u = to_f32(s[i]), v = to_f32(s[i + half]);
-        d[at(i)] = from_f32<OT>(u * cs - v * sn);
-        d[at(i + half)] = from_f32<OT>(v * cs + u * sn);
+        const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+        const float u = to_f32(s[ia]), v = to_f32(s[ib]);
+        d[at(ia)] = from_f32<OT>(u * cs - v * sn);
+        d[at(ib)] = from_f32<OT>(v * cs + u * sn);
     }
     for (int i = rot_dims + lane; i < width; i += nl) d[at(i)] = from_f32<OT>(to_f32(s[i]));
 }
@@ -593,20 +607,21 @@ __global__ __launch_bounds__(64) void qkv_rotate_store_kernel(const T* __restric
                                                               const int* __restrict__ tok_slot,
                                                               const float* __restrict__ inv_freq, float mag,
                                                               T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv,
-                                                              int pool_hdk, int pool_hdv) {
+                                                              int pool_hdk, int pool_hdv, int interleaved) {
     const long t = blockIdx.x;
     const int y = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[t];
     const T* row = qkv + t * ld;
     if (y < nh) {
-        rotate_run(row + (long)y * dk, q_out + (t * nh + y) * dk, dk, rot_dims, pos, inv_freq, mag, DST_ROWS, 0, lane, 64);
+        rotate_run(row + (long)y * dk, q_out + (t * nh + y) * dk, dk, rot_dims, pos, inv_freq, mag, DST_ROWS, 0, lane, 64,
+                   interleaved);
         return;
     }
     const long prow = paged_row(pv, tok_slot[t], pos);
     if (y < nh + nkv) {
         const int h = y - nh;
         rotate_run(row + (long)(nh + h) * dk, kpool + key_index(prow, h, nkv, pool_hdk), dk, rot_dims, pos, inv_freq, mag,
-                   DST_KEYS, 0, lane, 64);
+                   DST_KEYS, 0, lane, 64, interleaved);
     } else {
         const int h = y - nh - nkv;
         rotate_run(row + (long)(nh + nkv) * dk + (long)h * dv, vpool + value_index(prow, h, nkv, pool_hdv), dv, 0, pos,
@@ -618,7 +633,7 @@ extern "C" const char* cpmcu_qkv_rotate_store(const void* qkv, long ld, int dtyp
                                               int dk, int dv, int rot_dims, const int* positions, const int* tok_slot,
                                               const float* inv_freq, float mag, void* kpool, void* vpool,
                                               const int* page_table, int table_width, int page_size, int pool_hdk,
-                                              int pool_hdv, int write_kv, hipStream_t stream) {
+                                              int pool_hdv, int write_kv, int interleaved, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "qkv_rotate_store: empty shape");
     CPMCU_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dk && (rot_dims == 0 || inv_freq),
                   "qkv_rotate_store: %d rotated features of %d", rot_dims, dk);
@@ -633,11 +648,12 @@ extern "C" const char* cpmcu_qkv_rotate_store(const void* qkv, long ld, int dtyp
     if (dtype == CPMCU_F32)
         qkv_rotate_store_kernel<float><<<grid, 64, 0, stream>>>((const float*)qkv, ld, (float*)q_out, nh, nkv, dk, dv, rot_dims,
                                                                 positions, tok_slot, inv_freq, mag, (float*)kpool,
-                                                                (float*)vpool, pv, pool_hdk, pool_hdv);
+                                                                (float*)vpool, pv, pool_hdk, pool_hdv, interleaved);
     else if (dtype == CPMCU_BF16)
         qkv_rotate_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)qkv, ld, (bf16_t*)q_out, nh, nkv, dk, dv,
                                                                  rot_dims, positions, tok_slot, inv_freq, mag,
-                                                                 (bf16_t*)kpool, (bf16_t*)vpool, pv, pool_hdk, pool_hdv);
+                                                                 (bf16_t*)kpool, (bf16_t*)vpool, pv, pool_hdk, pool_hdv,
+                                                                 interleaved);
     else
         CPMCU_FAIL("qkv_rotate_store: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("qkv_rotate_store");
@@ -652,14 +668,16 @@ extern "C" const char* cpmcu_qkv_rotate_store(const void* qkv, long ld, int dtyp
 //   * with values_from_keys the row holds no v: the value pages receive k as projected (with its bias, before norm
 //     and rotation), so dv == dk;
 //   * with norm_after q and k heads are rotated first and then divided by their root mean square (times the
-//     weight, if one is given).
-template <typename T>
+//     weight, if one is given);
+//   * with interleaved the rotation pairs neighbouring features (2i, 2i + 1) instead of (i, i + rot_dims/2).
+// The projection's rows may be float where the cache is bfloat16 (rows that a convolution wrote).
+template <typename IT, typename T>
 __global__ __launch_bounds__(64) void qkv_norm_rotate_store_kernel(
-    const T* __restrict__ qkv, long ld, const float* __restrict__ bias, T* __restrict__ q_out, int nh, int nkv, int dk,
+    const IT* __restrict__ qkv, long ld, const float* __restrict__ bias, T* __restrict__ q_out, int nh, int nkv, int dk,
     int dv, int rot_dims, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
     int values_from_keys, const int* __restrict__ positions, const int* __restrict__ tok_slot,
     const float* __restrict__ inv_freq, float mag, T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv,
-    int pool_hdk, int pool_hdv, int norm_after) {
+    int pool_hdk, int pool_hdv, int norm_after, int interleaved) {
     __shared__ float hs[AG_MAX_HD];
     const long t = blockIdx.x;
     const int y = blockIdx.y, lane = threadIdx.x;
@@ -668,7 +686,7 @@ __global__ __launch_bounds__(64) void qkv_norm_rotate_store_kernel(
     const int h = is_q ? y : (is_k ? y - nh : y - nh - nkv);
     const int width = (is_q || is_k) ? dk : dv;
     const long col = is_q ? (long)h * dk : (is_k ? (long)(nh + h) * dk : (long)(nh + nkv) * dk + (long)h * dv);
-    const T* src = qkv + t * ld + col;
+    const IT* src = qkv + t * ld + col;
     const long prow = is_q ? 0 : paged_row(pv, tok_slot[t], pos);
     if (!is_q && !is_k) {               // a value head of its own: copied as it is
         T* vd = vpool + value_index(prow, h, nkv, pool_hdv);
@@ -693,9 +711,10 @@ __global__ __launch_bounds__(64) void qkv_norm_rotate_store_kernel(
         for (int i = lane; i < half; i += 64) {
             const float ang = (float)pos * inv_freq[i];
             const float cs = cosf(ang) * mag, sn = sinf(ang) * mag;
-            const float u = hs[i], v = hs[i + half];
-            hs[i] = u * cs - v * sn;
-            hs[i + half] = v * cs + u * sn;
+            const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+            const float u = hs[ia], v = hs[ib];
+            hs[ia] = u * cs - v * sn;
+            hs[ib] = v * cs + u * sn;
         }
         __syncthreads();
         float s2 = 0.f;
@@ -708,8 +727,9 @@ __global__ __launch_bounds__(64) void qkv_norm_rotate_store_kernel(
         for (int i = lane; i < width; i += 64) hs[i] = hs[i] * r * nw[i];
     }
     __syncthreads();
-    if (is_q) rotate_run(hs, q_out + (t * nh + h) * dk, dk, rot_dims, pos, inv_freq, mag, DST_ROWS, 0, lane, 64);
-    else rotate_run(hs, kpool + key_index(prow, h, nkv, pool_hdk), dk, rot_dims, pos, inv_freq, mag, DST_KEYS, 0, lane, 64);
+    if (is_q) rotate_run(hs, q_out + (t * nh + h) * dk, dk, rot_dims, pos, inv_freq, mag, DST_ROWS, 0, lane, 64, interleaved);
+    else rotate_run(hs, kpool + key_index(prow, h, nkv, pool_hdk), dk, rot_dims, pos, inv_freq, mag, DST_KEYS, 0, lane, 64,
+                    interleaved);
 }
 
 extern "C" const char* cpmcu_qkv_norm_rotate_store(const void* qkv, long ld, int dtype, const float* bias, void* q_out,
@@ -718,7 +738,8 @@ extern "C" const char* cpmcu_qkv_norm_rotate_store(const void* qkv, long ld, int
                                                    int values_from_keys, const int* positions, const int* tok_slot,
                                                    const float* inv_freq, float mag, void* kpool, void* vpool,
                                                    const int* page_table, int table_width, int page_size, int pool_hdk,
-                                                   int pool_hdv, int write_kv, int norm_after, hipStream_t stream) {
+                                                   int pool_hdv, int write_kv, int norm_after, int interleaved, int in_dtype,
+                                                   hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "qkv_norm_rotate_store: empty shape");
     CPMCU_REQUIRE(dk <= AG_MAX_HD && dv <= AG_MAX_HD, "qkv_norm_rotate_store: key size %d / value size %d (up to %d are taken)",
                   dk, dv, AG_MAX_HD);
@@ -734,17 +755,16 @@ extern "C" const char* cpmcu_qkv_norm_rotate_store(const void* qkv, long ld, int
     CPMCU_REQUIRE(heads <= 65535, "qkv_norm_rotate_store: %d heads exceed the launch grid", heads);
     PagedView pv{page_table, table_width, page_size};
     dim3 grid(n, heads);
-    if (dtype == CPMCU_F32)
-        qkv_norm_rotate_store_kernel<float><<<grid, 64, 0, stream>>>(
-            (const float*)qkv, ld, bias, (float*)q_out, nh, nkv, dk, dv, rot_dims, q_norm_w, k_norm_w, eps, values_from_keys,
-            positions, tok_slot, inv_freq, mag, (float*)kpool, (float*)vpool, pv, pool_hdk, pool_hdv, norm_after);
-    else if (dtype == CPMCU_BF16)
-        qkv_norm_rotate_store_kernel<bf16_t><<<grid, 64, 0, stream>>>(
-            (const bf16_t*)qkv, ld, bias, (bf16_t*)q_out, nh, nkv, dk, dv, rot_dims, q_norm_w, k_norm_w, eps,
-            values_from_keys, positions, tok_slot, inv_freq, mag, (bf16_t*)kpool, (bf16_t*)vpool, pv, pool_hdk, pool_hdv,
-            norm_after);
-    else
-        CPMCU_FAIL("qkv_norm_rotate_store: unknown dtype %d", dtype);
+#define LAUNCH(ITv, Tv)                                                                                              \
+    qkv_norm_rotate_store_kernel<ITv, Tv><<<grid, 64, 0, stream>>>(                                                  \
+        (const ITv*)qkv, ld, bias, (Tv*)q_out, nh, nkv, dk, dv, rot_dims, q_norm_w, k_norm_w, eps, values_from_keys, \
+        positions, tok_slot, inv_freq, mag, (Tv*)kpool, (Tv*)vpool, pv, pool_hdk, pool_hdv, norm_after, interleaved)
+    // dtype: the cache's and q_out's element type; in_dtype: the projection rows' (float rows may feed a bfloat16 cache)
+    if (dtype == CPMCU_F32 && in_dtype == CPMCU_F32) LAUNCH(float, float);
+    else if (dtype == CPMCU_BF16 && in_dtype == CPMCU_BF16) LAUNCH(bf16_t, bf16_t);
+    else if (dtype == CPMCU_BF16 && in_dtype == CPMCU_F32) LAUNCH(float, bf16_t);
+    else CPMCU_FAIL("qkv_norm_rotate_store: unsupported dtypes in=%d out=%d", in_dtype, dtype);
+#undef LAUNCH
     CPMCU_LAUNCH_CHECK("qkv_norm_rotate_store");
     return nullptr;
 }

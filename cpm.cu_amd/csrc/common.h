@@ -43,11 +43,21 @@ template <typename T> __host__ __device__ inline T from_f32(float f);
 template <> __host__ __device__ inline float from_f32<float>(float f) { return f; }
 template <> __host__ __device__ inline bf16_t from_f32<bf16_t>(float f) { return f32_to_bf16(f); }
 
-// Nonlinearity of a gated feed-forward's gate, act(g) * up.  Both kinds are g * sigmoid(s(g)): SiLU with s(g) = g,
-// the tanh form of GELU with s(g) = 2 sqrt(2/pi) (g + 0.044715 g^3), since 0.5 (1 + tanh z) = sigmoid(2 z).
-enum { CPMCU_ACT_SILU = 0, CPMCU_ACT_GELU_TANH = 1 };
+// Nonlinearity of a gated feed-forward's gate, act(g) * up.  All kinds are g * sigmoid(s(g)): SiLU with s(g) = g,
+// the tanh form of GELU with s(g) = 2 sqrt(2/pi) (g + 0.044715 g^3), since 0.5 (1 + tanh z) = sigmoid(2 z), and the
+// clamped swish with s(g) = 1.702 g, whose pair is first cut off at a limit and whose up half is raised by one:
+// g <- min(g, limit), up <- clamp(up, -limit, limit) + 1 (gate_prepare, a no-op for the other kinds).
+enum { CPMCU_ACT_SILU = 0, CPMCU_ACT_GELU_TANH = 1, CPMCU_ACT_CLAMPED_SWISH = 2 };
+#define CPMCU_ACT_KNOWN(act) ((act) >= CPMCU_ACT_SILU && (act) <= CPMCU_ACT_CLAMPED_SWISH)
 __host__ __device__ inline float gate_arg(float g, int act) {
-    return act == CPMCU_ACT_GELU_TANH ? 1.5957691216057308f * (g + 0.044715f * g * g * g) : g;
+    return act == CPMCU_ACT_GELU_TANH ? 1.5957691216057308f * (g + 0.044715f * g * g * g)
+                                      : (act == CPMCU_ACT_CLAMPED_SWISH ? 1.702f * g : g);
+}
+__device__ inline void gate_prepare(float& g, float& up, int act, float limit) {
+    if (act == CPMCU_ACT_CLAMPED_SWISH) {
+        g = fminf(g, limit);
+        up = fminf(fmaxf(up, -limit), limit) + 1.0f;
+    }
 }
 __device__ inline float gate_act(float g, int act) { return g / (1.0f + expf(-gate_arg(g, act))); }
 

@@ -34,6 +34,58 @@ extern "C" const char* cpmcu_embed(const void* table, int dtype, const int* ids,
     return nullptr;
 }
 
+// ---------------------------------------------------------------------------
+// A second table read by a hash of the previous token and the current one, added to the embedding:
+// out[r,:] += float(table[(prev * mul_prev + ids[r] * mul_cur) mod buckets, :]); a sequence's first token (position
+// 0) reads row `buckets`, the table's last.  The previous token of a row is the row before it in the packed batch, or,
+// for the first row a sequence brings in this step, what the sequence's slot remembers (prev_state int32 [slots]).
+// A second launch (bigram_remember_kernel) then moves every slot on to the last token its sequence brought.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void bigram_add_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                  const int* __restrict__ positions, const int* __restrict__ tok_slot,
+                                  const int* __restrict__ prev_state, float* __restrict__ out, int H, long buckets,
+                                  long mul_prev, long mul_cur) {
+    const long r = blockIdx.x;
+    long row = buckets;
+    if (positions[r] > 0) {
+        const int slot = tok_slot[r];
+        const int prev = (r > 0 && tok_slot[r - 1] == slot) ? ids[r - 1] : prev_state[slot];
+        row = ((long)prev * mul_prev + (long)ids[r] * mul_cur) % buckets;
+    }
+    const T* src = table + row * H;
+    float* dst = out + r * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] += to_f32(src[c]);
+}
+
+__global__ void bigram_remember_kernel(const int* __restrict__ ids, const int* __restrict__ cu_q,
+                                       const int* __restrict__ seq_slot, int* __restrict__ prev_state, int n_seqs) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < n_seqs && cu_q[b + 1] > cu_q[b]) prev_state[seq_slot[b]] = ids[cu_q[b + 1] - 1];
+}
+
+extern "C" const char* cpmcu_bigram_add(const void* table, int dtype, const int* ids, const int* positions,
+                                        const int* tok_slot, int* prev_state, const int* cu_q, const int* seq_slot,
+                                        float* out, int n, int n_seqs, int H, long buckets, long mul_prev, long mul_cur,
+                                        int remember, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && n_seqs > 0 && buckets > 0, "bigram_add: empty shape n=%d H=%d buckets=%ld", n, H, buckets);
+    CPMCU_REQUIRE(mul_prev >= 0 && mul_cur >= 0, "bigram_add: multipliers must not be negative");
+    CPMCU_REQUIRE(dtype == CPMCU_F32 || dtype == CPMCU_BF16, "bigram_add: unknown dtype %d", dtype);
+    const int block = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+    if (dtype == CPMCU_F32)
+        bigram_add_kernel<float><<<n, block, 0, stream>>>((const float*)table, ids, positions, tok_slot, prev_state, out, H,
+                                                          buckets, mul_prev, mul_cur);
+    else
+        bigram_add_kernel<bf16_t><<<n, block, 0, stream>>>((const bf16_t*)table, ids, positions, tok_slot, prev_state, out,
+                                                           H, buckets, mul_prev, mul_cur);
+    CPMCU_LAUNCH_CHECK("bigram_add");
+    if (remember) {
+        bigram_remember_kernel<<<(n_seqs + 63) / 64, 64, 0, stream>>>(ids, cu_q, seq_slot, prev_state, n_seqs);
+        CPMCU_LAUNCH_CHECK("bigram_remember");
+    }
+    return nullptr;
+}
+
 // logits <- cap * tanh(logits / cap), in place (a soft cap on the head's output)
 __global__ void softcap_kernel(float* __restrict__ x, long total, float cap) {
     const float inv = 1.0f / cap;
@@ -281,13 +333,14 @@ extern "C" const char* cpmcu_add_norm_columns(float* x, const void* branch, int 
 // (reference: src/model/activation.cuh:6-18, gate columns first, then up)
 // ---------------------------------------------------------------------------
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, long n, int I, int act) {
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, long n, int I, int act, float limit) {
     const long total = n * I;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
         const long r = i / I;
         const int c = (int)(i - r * I);
-        const float g = to_f32(gu[r * 2 * I + c]);
-        const float u = to_f32(gu[r * 2 * I + I + c]);
+        float g = to_f32(gu[r * 2 * I + c]);
+        float u = to_f32(gu[r * 2 * I + I + c]);
+        gate_prepare(g, u, act, limit);
         out[i] = from_f32<T>(gate_act(g, act) * u);
     }
 }
@@ -298,7 +351,7 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, l
 // (2^-22 relative; the 32-bit engine's kernel above keeps expf and a true division).
 template <int U>
 __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
-                                                              long n, int I, int act) {
+                                                              long n, int I, int act, float limit) {
     const int I8 = I / 8;
     const long total = n * I8;
     const long base = (long)blockIdx.x * (256 * U) + threadIdx.x;
@@ -320,8 +373,10 @@ __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __re
         uint32_t ow[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
-            const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+            float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+            float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+            gate_prepare(g0, u0, act, limit);
+            gate_prepare(g1, u1, act, limit);
             const float s0 = g0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * gate_arg(g0, act)));
             const float s1 = g1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * gate_arg(g1, act)));
             const bf16_t a = f32_to_bf16(s0 * u0);
@@ -332,20 +387,21 @@ __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __re
     }
 }
 
-extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int n, int I, int act, hipStream_t stream) {
+extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int n, int I, int act, float limit,
+                                      hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && I > 0, "silu_mul: empty shape n=%d I=%d", n, I);
-    CPMCU_REQUIRE(act == CPMCU_ACT_SILU || act == CPMCU_ACT_GELU_TANH, "silu_mul: unknown nonlinearity %d", act);
+    CPMCU_REQUIRE(CPMCU_ACT_KNOWN(act), "silu_mul: unknown nonlinearity %d", act);
     if (dtype == CPMCU_BF16 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
         const long total8 = (long)n * (I / 8);
         // many rows: 4 pieces a thread in flight; few: one, for more workgroups
         if (total8 >= 4L * 256 * 2048) {
             const long wgs = (total8 + 4 * 256 - 1) / (4 * 256);
             CPMCU_REQUIRE(wgs <= 0x7fffffffL, "silu_mul: %d rows of %d columns exceed the launch grid", n, I);
-            silu_mul_bf16x8_kernel<4><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I, act);
+            silu_mul_bf16x8_kernel<4><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I, act, limit);
         } else {
             const long wgs = (total8 + 255) / 256;
             CPMCU_REQUIRE(wgs <= 0x7fffffffL, "silu_mul: %d rows of %d columns exceed the launch grid", n, I);
-            silu_mul_bf16x8_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I, act);
+            silu_mul_bf16x8_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I, act, limit);
         }
         CPMCU_LAUNCH_CHECK("silu_mul");
         return nullptr;
@@ -354,9 +410,9 @@ extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int 
     const int block = 256;
     const int grid = (int)((total + block - 1) / block < 65535 * 16 ? (total + block - 1) / block : 65535 * 16);
     if (dtype == CPMCU_F32)
-        silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, n, I, act);
+        silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, n, I, act, limit);
     else if (dtype == CPMCU_BF16)
-        silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I, act);
+        silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I, act, limit);
     else
         CPMCU_FAIL("silu_mul: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("silu_mul");

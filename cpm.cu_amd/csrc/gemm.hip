@@ -270,7 +270,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
                                                              OT* __restrict__ Y, long ldy, int M, int N, int K, int KS,
                                                              float alpha, int I, long part_stride,
                                                              const float* __restrict__ row_ss, int ss_slices,
-                                                             float eps, int act) {
+                                                             float eps, int act, float act_limit) {
     static_assert(MODE != 2 || SPW == 2, "gated output pairs a gate strip with an up strip");
     // whether the x operands are read from LDS a step ahead (below): it pays for 4 tiles of rows in the split and
     // plain products (64 rows, us without/with: q/k/v 17.0/14.3, down 31.0/28.9, head 134/130, o 11.7/12.0), not
@@ -456,7 +456,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
             for (int i = 0; i < 4; ++i) {
                 const int col = out_base[0] + 4 * g + i;
                 if (col < I) {
-                    const float gt = acc[0][t][i] * rs_t, up = acc[SPW - 1][t][i] * rs_t;
+                    float gt = acc[0][t][i] * rs_t, up = acc[SPW - 1][t][i] * rs_t;
+                    gate_prepare(gt, up, act, act_limit);
                     Yp[(long)tok * ldy + col] = from_f32<OT>(gate_act(gt, act) * up);
                 }
             }
@@ -483,8 +484,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
 extern "C" const char* cpmcu_gemm_skinny(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
                                          int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
                                          int tiled, const float* row_ss, int ss_slices, float eps, int act,
-                                         hipStream_t stream) {
-    CPMCU_REQUIRE(act == CPMCU_ACT_SILU || act == CPMCU_ACT_GELU_TANH, "gemm_skinny: unknown nonlinearity %d", act);
+                                         float act_limit, hipStream_t stream) {
+    CPMCU_REQUIRE(CPMCU_ACT_KNOWN(act), "gemm_skinny: unknown nonlinearity %d", act);
     CPMCU_REQUIRE(M > 0 && M <= 64, "gemm_skinny: %d rows (1..64 are taken; more rows belong to the tiled product)", M);
     CPMCU_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: K=%d must be a positive multiple of 8 (N=%d)", K, N);
     CPMCU_REQUIRE(ldx % 8 == 0 && ldx >= K && (tiled || (ldw % 8 == 0 && ldw >= K)),
@@ -508,11 +509,11 @@ extern "C" const char* cpmcu_gemm_skinny(const void* X, long ldx, const void* W,
         if (tiled)                                                                                                \
             gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, true><<<grid, NW * 64, 0, stream>>>(                      \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
-                row_ss, ss_slices, eps, act);                                                                     \
+                row_ss, ss_slices, eps, act, act_limit);                                                               \
         else                                                                                                      \
             gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, false><<<grid, NW * 64, 0, stream>>>(                     \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
-                row_ss, ss_slices, eps, act);                                                                     \
+                row_ss, ss_slices, eps, act, act_limit);                                                               \
     } while (0)
 #define BY_MT(MODEv, OT, SPW, NW)                     \
     do {                                              \

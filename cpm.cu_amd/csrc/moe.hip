@@ -1,13 +1,15 @@
 // A feed-forward of routed experts, for steps of any number of tokens and both element types:
 //
 //  * moe_logits_kernel, moe_select_kernel: router logits z = Wr h in float (Wr float [E, H]), a wavefront a row,
-//    into scratch; then, a wavefront a token: s = softmax(z); choice scores c = s +
-//    correction; the experts form `n_groups` equal groups of neighbours, a group's score is its largest c, and only
-//    experts of the `keep_groups` best groups may be chosen (n_groups = 1: any); the `top` largest c are chosen
-//    (ties: the lower index), their weights are s / (sum of the chosen s + 1e-20).  With w_sg (float [H]) it also
+//    into scratch; then, a wavefront a token: s = softmax(z) over the experts, or sigmoid(z) of each (score_fn);
+//    choice scores c = s + correction; the experts form `n_groups` equal groups of neighbours, a group's score is
+//    its largest c, or the sum of its two largest (group_fn), and only experts of the `keep_groups` best groups may be
+//    chosen (n_groups = 1: any; the others' c count as -inf); the `top` largest c are chosen (ties: the lower index),
+//    their weights are s / (sum of the chosen s + 1e-20) * weight_scale.  With w_sg (float [H]) it also
 //    gives sigmoid(w_sg . h), the gate of an expert that every token uses.
-//  * moe_gated_kernel: act[t, k, :] = silu(Wg_e h_t) * (Wu_e h_t) for the k-th chosen expert e of token t; the
-//    experts' gate and up rows are stacked: wgu [E, 2F, H], gate rows first.
+//  * moe_gated_kernel: act[t, k, :] = act(Wg_e h_t) * (Wu_e h_t) for the k-th chosen expert e of token t (the
+//    nonlinearities of common.h: SiLU, or the clamped swish with its limit); the experts' gate and up rows are
+//    stacked: wgu [E, 2F, H], gate rows first.
 //  * moe_down_kernel: out[t] = sum_k w[t, k] Wd_e act[t, k] (+ sg[t] * shared[t]); wd [E, H, F]; float out.
 //
 // A wavefront owns output rows and its lanes stride over the input features (16-byte loads when the rows are
@@ -15,6 +17,8 @@
 #include "common.h"
 
 #define MOE_MAX_EXPERTS 1024
+enum { MOE_SCORE_SOFTMAX = 0, MOE_SCORE_SIGMOID = 1 };
+enum { MOE_GROUP_MAX = 0, MOE_GROUP_TOP2_SUM = 1 };
 
 template <typename T> struct Vec8;
 template <> struct Vec8<bf16_t> { typedef uint4 type; };
@@ -80,7 +84,8 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const T* __restrict__ h
 __global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict__ logits,
                                                         const float* __restrict__ correction, int has_sg, int E,
                                                         int n_groups, int keep_groups, int top, int* __restrict__ idx_out,
-                                                        float* __restrict__ w_out, float* __restrict__ sg_out) {
+                                                        float* __restrict__ w_out, float* __restrict__ sg_out,
+                                                        int score_fn, int group_fn, float weight_scale) {
     __shared__ float z[MOE_MAX_EXPERTS];      // logits, then softmax scores
     __shared__ float c[MOE_MAX_EXPERTS];      // choice scores; -inf once an expert is chosen or shut out
     __shared__ float gs[MOE_MAX_EXPERTS];     // group scores
@@ -88,31 +93,47 @@ __global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict_
     const int lane = threadIdx.x;
     const float* zr = logits + t * (E + 1);
     if (has_sg && lane == 0) sg_out[t] = 1.0f / (1.0f + expf(-zr[E]));
-    float mx = -INFINITY;
-    for (int e = lane; e < E; e += 64) {
-        z[e] = zr[e];
-        mx = fmaxf(mx, z[e]);
-    }
-    mx = wave_max(mx);
-    float sum = 0.f;
-    for (int e = lane; e < E; e += 64) {
-        const float p = expf(z[e] - mx);
-        z[e] = p;
-        sum += p;
-    }
-    sum = wave_sum(sum);
-    const float inv = 1.0f / sum;
-    for (int e = lane; e < E; e += 64) {
-        z[e] *= inv;
-        c[e] = z[e] + (correction ? correction[e] : 0.f);
+    if (score_fn == MOE_SCORE_SIGMOID) {
+        for (int e = lane; e < E; e += 64) {
+            z[e] = 1.0f / (1.0f + expf(-zr[e]));
+            c[e] = z[e] + (correction ? correction[e] : 0.f);
+        }
+    } else {
+        float mx = -INFINITY;
+        for (int e = lane; e < E; e += 64) {
+            z[e] = zr[e];
+            mx = fmaxf(mx, z[e]);
+        }
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += 64) {
+            const float p = expf(z[e] - mx);
+            z[e] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum);
+        const float inv = 1.0f / sum;
+        for (int e = lane; e < E; e += 64) {
+            z[e] *= inv;
+            c[e] = z[e] + (correction ? correction[e] : 0.f);
+        }
     }
     __builtin_amdgcn_wave_barrier();
     if (n_groups > 1) {
         const int per = E / n_groups;
         for (int g = lane; g < n_groups; g += 64) {
-            float b = -INFINITY;
-            for (int i = 0; i < per; ++i) b = fmaxf(b, c[g * per + i]);
-            gs[g] = b;
+            // the largest and the second largest choice score of the group
+            float b = -INFINITY, b2 = -INFINITY;
+            for (int i = 0; i < per; ++i) {
+                const float v = c[g * per + i];
+                if (v > b) {
+                    b2 = b;
+                    b = v;
+                } else if (v > b2) {
+                    b2 = v;
+                }
+            }
+            gs[g] = (group_fn == MOE_GROUP_TOP2_SUM && per > 1) ? b + b2 : b;
         }
         __builtin_amdgcn_wave_barrier();
         // the best groups, one a turn, are marked with +inf; afterwards every other group's experts are shut out
@@ -149,13 +170,17 @@ __global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict_
         }
         __builtin_amdgcn_wave_barrier();
     }
-    const float norm = 1.0f / (chosen_sum + 1e-20f);
+    const float norm = weight_scale / (chosen_sum + 1e-20f);
     for (int r = lane; r < top; r += 64) w_out[t * top + r] *= norm;
 }
 
 extern "C" const char* cpmcu_moe_route(const void* h, long ldh, int dtype, const float* wr, const float* correction,
                                        const float* w_sg, int n, int H, int E, int n_groups, int keep_groups, int top,
-                                       float* logits, int* idx_out, float* w_out, float* sg_out, hipStream_t stream) {
+                                       float* logits, int* idx_out, float* w_out, float* sg_out, int score_fn,
+                                       int group_fn, float weight_scale, hipStream_t stream) {
+    CPMCU_REQUIRE((score_fn == MOE_SCORE_SOFTMAX || score_fn == MOE_SCORE_SIGMOID) &&
+                  (group_fn == MOE_GROUP_MAX || group_fn == MOE_GROUP_TOP2_SUM),
+                  "moe_route: unknown score function %d or group score %d", score_fn, group_fn);
     CPMCU_REQUIRE(n > 0 && H > 0 && E > 0 && logits, "moe_route: empty shape");
     CPMCU_REQUIRE(E <= MOE_MAX_EXPERTS, "moe_route: %d experts (up to %d are taken)", E, MOE_MAX_EXPERTS);
     CPMCU_REQUIRE(n_groups >= 1 && E % n_groups == 0 && keep_groups >= 1 && keep_groups <= n_groups,
@@ -172,7 +197,7 @@ extern "C" const char* cpmcu_moe_route(const void* h, long ldh, int dtype, const
         CPMCU_FAIL("moe_route: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("moe_logits");
     moe_select_kernel<<<n, 64, 0, stream>>>(logits, correction, w_sg ? 1 : 0, E, n_groups, keep_groups, top, idx_out, w_out,
-                                            sg_out);
+                                            sg_out, score_fn, group_fn, weight_scale);
     CPMCU_LAUNCH_CHECK("moe_select");
     return nullptr;
 }
@@ -183,7 +208,7 @@ extern "C" const char* cpmcu_moe_route(const void* h, long ldh, int dtype, const
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gated_kernel(const T* __restrict__ h, long ldh, const T* __restrict__ wgu,
                                                         const int* __restrict__ idx, T* __restrict__ act, int H, int F,
-                                                        int top) {
+                                                        int top, int act_fn, float act_limit) {
     const long pair = blockIdx.x;
     const long t = pair / top;
     const int e = idx[pair];
@@ -196,22 +221,24 @@ __global__ __launch_bounds__(256) void moe_gated_kernel(const T* __restrict__ h,
     for (int r = 0; r < MOE_ROWS; ++r) {
         const int j = j0 + r;
         if (j >= F) break;
-        const float g = wave_sum(lane_dot<T, T>(wg + (long)j * H, hr, H, lane, vec));
-        const float u = wave_sum(lane_dot<T, T>(wg + (long)(F + j) * H, hr, H, lane, vec));
-        if (lane == 0) act[pair * F + j] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+        float g = wave_sum(lane_dot<T, T>(wg + (long)j * H, hr, H, lane, vec));
+        float u = wave_sum(lane_dot<T, T>(wg + (long)(F + j) * H, hr, H, lane, vec));
+        gate_prepare(g, u, act_fn, act_limit);
+        if (lane == 0) act[pair * F + j] = from_f32<T>(gate_act(g, act_fn) * u);
     }
 }
 
 extern "C" const char* cpmcu_moe_gated(const void* h, long ldh, int dtype, const void* wgu, const int* idx, void* act,
-                                       int n, int H, int F, int top, hipStream_t stream) {
+                                       int n, int H, int F, int top, int act_fn, float act_limit, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && H > 0 && F > 0 && top > 0, "moe_gated: empty shape");
+    CPMCU_REQUIRE(CPMCU_ACT_KNOWN(act_fn), "moe_gated: unknown nonlinearity %d", act_fn);
     const int fy = (F + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS);
     CPMCU_REQUIRE(fy <= 65535, "moe_gated: %d rows an expert exceed the launch grid", F);
     dim3 grid((unsigned)((long)n * top), fy);
     if (dtype == CPMCU_F32)
-        moe_gated_kernel<float><<<grid, 256, 0, stream>>>((const float*)h, ldh, (const float*)wgu, idx, (float*)act, H, F, top);
+        moe_gated_kernel<float><<<grid, 256, 0, stream>>>((const float*)h, ldh, (const float*)wgu, idx, (float*)act, H, F, top, act_fn, act_limit);
     else if (dtype == CPMCU_BF16)
-        moe_gated_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)wgu, idx, (bf16_t*)act, H, F, top);
+        moe_gated_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)wgu, idx, (bf16_t*)act, H, F, top, act_fn, act_limit);
     else
         CPMCU_FAIL("moe_gated: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("moe_gated");
@@ -324,7 +351,7 @@ __global__ __launch_bounds__(256) void moe_gated_mfma_kernel(const bf16_t* __res
                                                              const bf16_t* __restrict__ wgu, const int* __restrict__ rows,
                                                              const int* __restrict__ tile_expert,
                                                              const int* __restrict__ n_tiles, bf16_t* __restrict__ act,
-                                                             int H, int F, int top) {
+                                                             int H, int F, int top, int act_fn, float act_limit) {
     const int tile = blockIdx.y;
     if (tile >= *n_tiles) return;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -378,8 +405,9 @@ __global__ __launch_bounds__(256) void moe_gated_mfma_kernel(const bf16_t* __res
             for (int j = 0; j < 2; ++j) {
                 const int f = f0 + 16 * j + r;
                 if (f < F) {
-                    const float gt = acc[rt][j][i], up = acc[rt][2 + j][i];
-                    act[(long)p * F + f] = f32_to_bf16(gt / (1.0f + expf(-gt)) * up);
+                    float gt = acc[rt][j][i], up = acc[rt][2 + j][i];
+                    gate_prepare(gt, up, act_fn, act_limit);
+                    act[(long)p * F + f] = f32_to_bf16(gate_act(gt, act_fn) * up);
                 }
             }
         }
@@ -469,8 +497,9 @@ extern "C" const char* cpmcu_moe_experts_mfma(const void* h, long ldh, const voi
                                               const float* w, const void* shared, int shared_dtype, int shared_parts,
                                               long shared_stride, const float* sg, void* act, void* y, int* rows,
                                               int* tile_expert, int* n_tiles, int max_tiles, float* out, int n, int H,
-                                              int F, int E, int top, hipStream_t stream) {
+                                              int F, int E, int top, int act_fn, float act_limit, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && H > 0 && F > 0 && E > 0 && top > 0, "moe_experts_mfma: empty shape");
+    CPMCU_REQUIRE(CPMCU_ACT_KNOWN(act_fn), "moe_experts_mfma: unknown nonlinearity %d", act_fn);
     CPMCU_REQUIRE(E <= MOE_MAX_EXPERTS, "moe_experts_mfma: %d experts (up to %d are taken)", E, MOE_MAX_EXPERTS);
     CPMCU_REQUIRE(H % 8 == 0 && F % 8 == 0 && ldh % 8 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)wgu % 16 == 0 &&
                   (uintptr_t)wd % 16 == 0 && (uintptr_t)act % 16 == 0,
@@ -481,7 +510,7 @@ extern "C" const char* cpmcu_moe_experts_mfma(const void* h, long ldh, const voi
     moe_group_kernel<<<1, 1024, 0, stream>>>(idx, (int)pairs, E, rows, tile_expert, n_tiles, max_tiles);
     CPMCU_LAUNCH_CHECK("moe_group");
     moe_gated_mfma_kernel<<<dim3((F + 127) / 128, max_tiles), 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)wgu, rows,
-                                                                            tile_expert, n_tiles, (bf16_t*)act, H, F, top);
+                                                                            tile_expert, n_tiles, (bf16_t*)act, H, F, top, act_fn, act_limit);
     CPMCU_LAUNCH_CHECK("moe_gated_mfma");
     moe_down_mfma_kernel<<<dim3((H + 255) / 256, max_tiles), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)wd, rows,
                                                                            tile_expert, n_tiles, (bf16_t*)y, H, F);

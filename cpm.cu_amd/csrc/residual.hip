@@ -5,6 +5,9 @@
 //    that is a projection of those rows; [g1 | g2] are the columns of one product, [b1 | b2] its bias.  A and F
 //    may come as float partial sums [parts][n][H] of a split product; F (and its gate) may be absent.
 //  * bias_sum_kernel: out = sum of the parts + bias, for a consumer that knows nothing of biases.
+//  * scaled_branches_kernel: out = sa * wa[c] * (A + a_bias) + sf * wf[c] * (F + f_bias): two results that are added
+//    with a number each (two mixers side by side whose sum is weighted) and / or a weight a column each (a layer
+//    scale on the results of a parallel layer's two sub-layers); wa, wf, F may be absent.
 #include "common.h"
 
 template <typename GT, typename AT, typename FT>
@@ -107,5 +110,49 @@ extern "C" const char* cpmcu_sigmoid_gate(const void* a, const void* g, long ldg
     else
         CPMCU_FAIL("sigmoid_gate: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("sigmoid_gate");
+    return nullptr;
+}
+
+template <typename AT, typename FT>
+__global__ __launch_bounds__(256) void scaled_branches_kernel(const AT* __restrict__ a, int a_parts, long a_stride,
+                                                              const float* __restrict__ a_bias,
+                                                              const float* __restrict__ wa, float sa,
+                                                              const FT* __restrict__ f, int f_parts, long f_stride,
+                                                              const float* __restrict__ f_bias,
+                                                              const float* __restrict__ wf, float sf,
+                                                              float* __restrict__ out, long total, int H) {
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+        const int c = (int)(i % H);
+        float av = a_bias ? a_bias[c] : 0.f;
+        for (int p = 0; p < a_parts; ++p) av += to_f32(a[(long)p * a_stride + i]);
+        float v = sa * (wa ? wa[c] : 1.0f) * av;
+        if (f) {
+            float fv = f_bias ? f_bias[c] : 0.f;
+            for (int p = 0; p < f_parts; ++p) fv += to_f32(f[(long)p * f_stride + i]);
+            v += sf * (wf ? wf[c] : 1.0f) * fv;
+        }
+        out[i] = v;
+    }
+}
+
+extern "C" const char* cpmcu_scaled_branches(const void* a, int a_dtype, int a_parts, long a_stride, const float* a_bias,
+                                             const float* wa, float sa, const void* f, int f_dtype, int f_parts,
+                                             long f_stride, const float* f_bias, const float* wf, float sf, float* out,
+                                             int n, int H, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && a && a_parts >= 1 && (!f || f_parts >= 1), "scaled_branches: empty shape");
+    const long total = (long)n * H;
+    const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    const int fd = f ? f_dtype : a_dtype;
+#define LAUNCH(AT, FT)                                                                                             \
+    scaled_branches_kernel<AT, FT><<<blocks, 256, 0, stream>>>((const AT*)a, a_parts, a_stride, a_bias, wa, sa,       \
+                                                               (const FT*)f, f_parts, f_stride, f_bias, wf, sf, out, \
+                                                               total, H)
+    if (a_dtype == CPMCU_F32 && fd == CPMCU_F32) LAUNCH(float, float);
+    else if (a_dtype == CPMCU_BF16 && fd == CPMCU_F32) LAUNCH(bf16_t, float);
+    else if (a_dtype == CPMCU_F32 && fd == CPMCU_BF16) LAUNCH(float, bf16_t);
+    else if (a_dtype == CPMCU_BF16 && fd == CPMCU_BF16) LAUNCH(bf16_t, bf16_t);
+    else CPMCU_FAIL("scaled_branches: unsupported dtypes a=%d f=%d", a_dtype, fd);
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("scaled_branches");
     return nullptr;
 }

@@ -164,7 +164,8 @@ extern "C" const char* cpmcu_proj_add_norm(const void* A, long lda, const void* 
 template <int PF, int NW, int MT>
 __global__ __launch_bounds__(NW * 64) void gated_strip_kernel(
     const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict__ W, int M, int I, int K,
-    bf16_t* __restrict__ out, const float* __restrict__ row_ss, int ss_slices, float eps, int act) {
+    bf16_t* __restrict__ out, const float* __restrict__ row_ss, int ss_slices, float eps, int act,
+    float act_limit) {
     __shared__ float red[NW - 1][2][MT][4][64];
     __shared__ float rs_s[MT * 16];
     const int strip = blockIdx.x;
@@ -247,6 +248,7 @@ __global__ __launch_bounds__(NW * 64) void gated_strip_kernel(
                 up += red[w][1][t][i][lane];
             }
             gt *= rs; up *= rs;
+            gate_prepare(gt, up, act, act_limit);
             o[i] = f32_to_bf16(gate_act(gt, act) * up).v;
         }
         if (tok < M && col < I) *(uint2*)(out + (long)tok * I + col) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
@@ -256,8 +258,9 @@ __global__ __launch_bounds__(NW * 64) void gated_strip_kernel(
 // a [M, K] bf16, W tiled [2 I, K], out [M, I] bf16; row_ss (or null): sums of squares [M][ss_slices] of a norm
 // cut by columns, whose row factor rsqrt(sum / K + eps) the rows of both products are multiplied by
 extern "C" const char* cpmcu_gated_strip(const void* A, long lda, const void* W, int M, int I, int K, void* out,
-                                         const float* row_ss, int ss_slices, float eps, int act, hipStream_t stream) {
-    CPMCU_REQUIRE(act == CPMCU_ACT_SILU || act == CPMCU_ACT_GELU_TANH, "gated_strip: unknown nonlinearity %d", act);
+                                         const float* row_ss, int ss_slices, float eps, int act, float act_limit,
+                                         hipStream_t stream) {
+    CPMCU_REQUIRE(CPMCU_ACT_KNOWN(act), "gated_strip: unknown nonlinearity %d", act);
     CPMCU_REQUIRE(M > 0 && M <= 16, "gated_strip: %d tokens (1..16 are taken; more go through the skinny product)", M);
     CPMCU_REQUIRE(I > 0 && I % 16 == 0 && K > 0 && K % 8 == 0 && lda % 8 == 0 && lda >= K,
                   "gated_strip: %d gate rows must be a multiple of 16, K=%d and the row stride %ld multiples of 8", I, K, lda);
@@ -265,7 +268,7 @@ extern "C" const char* cpmcu_gated_strip(const void* A, long lda, const void* W,
     CPMCU_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)out % 8 == 0),
                   "gated_strip: operands must be 16-byte aligned");
     gated_strip_kernel<4, 4, 1><<<I / 16, 256, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, M, I, K, (bf16_t*)out,
-                                                           row_ss, ss_slices, eps, act);
+                                                           row_ss, ss_slices, eps, act, act_limit);
     CPMCU_LAUNCH_CHECK("gated_strip");
     return nullptr;
 }

@@ -4,3 +4,4 @@ from . import minicpm
 from . import duvulix
 from . import gumodra
 from . import sagedra
+from . import nelutar

@@ -62,6 +62,11 @@ class DecoderModel(Part):
         self.n_cache_entries = (max(written) + 1) if written else 0
         if written != set(range(self.n_cache_entries)):
             raise ValueError("cache entries of the schedule must be numbered 0..n-1 without gaps")
+        # an embedding that keeps something per sequence (the previous token) owns one more entry, behind the runs'
+        self.embedding_entry = None
+        needs = getattr(self.embedding, "cache_needs", None)
+        if needs is not None and needs() is not None:
+            self.embedding_entry = self.n_cache_entries
 
     @property
     def vocab_size(self) -> int:
@@ -76,12 +81,17 @@ class DecoderModel(Part):
         for r in self.schedule:
             if r.writes_cache:
                 needs[r.cache] = self.layers[r.layer].mixer.cache_needs()
+        if self.embedding_entry is not None:
+            needs.append(self.embedding.cache_needs())
         return needs  # type: ignore[return-value]
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """float32 logits [R, V] at ctx.logit_rows; the step's tokens enter the cache."""
         with ctx.timed("embed"):
-            x = self.embedding.forward(ctx)
+            if self.embedding_entry is not None:
+                x = self.embedding.forward(ctx, ctx.cache.view(self.embedding_entry))
+            else:
+                x = self.embedding.forward(ctx)
             if self.streams:
                 lanes = ctx.ws.get("residual.streams", (self.streams,) + tuple(x.shape), torch.float32)
                 ops.streams_fill(x, lanes)

@@ -172,26 +172,38 @@ def add_norm_columns(x: torch.Tensor, branch: Optional[torch.Tensor], branch_sca
                                                  c_int(H), _stream()))
 
 
-GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "clamped_swish": 2}
 
 
-def _act(activation: str) -> int:
-    try:
-        return GATE_ACTIVATIONS[activation]
-    except KeyError:
-        raise KernelError(f"gate nonlinearity '{activation}' is not supported ({sorted(GATE_ACTIVATIONS)})") from None
+def gate_activation(activation):
+    """(name, limit) of a gated pair's nonlinearity given as a name or as (name, limit).  'clamped_swish' is the one
+    with a limit: g <- min(g, limit), up <- clamp(up, -limit, limit); the pair's product is g sigmoid(1.702 g) (up + 1)."""
+    name, limit = activation if isinstance(activation, (tuple, list)) else (activation, 0.0)
+    if name not in GATE_ACTIVATIONS:
+        raise KernelError(f"gate nonlinearity '{name}' is not supported ({sorted(GATE_ACTIVATIONS)})")
+    limit = float(limit or 0.0)
+    if name == "clamped_swish" and not limit > 0:
+        raise KernelError(f"gate nonlinearity 'clamped_swish' needs a positive limit, got {limit}")
+    return name, limit
 
 
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu"):
+def _act(activation):
+    """(c_int code, c_float limit) for the kernels."""
+    name, limit = gate_activation(activation)
+    return c_int(GATE_ACTIVATIONS[name]), c_float(limit)
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, activation="silu"):
     """out[r,c] = act(gate_up[r,c]) * gate_up[r,c+I];  gate_up [n,2I], out [n,I]; act is SiLU or, with
-    activation 'gelu_tanh', 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))."""
+    activation 'gelu_tanh', 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))), or ('clamped_swish', limit)
+    (gate_activation)."""
     _need(gate_up, "silu_mul input", shape=(None, None))
     n, two_i = gate_up.shape
     if two_i % 2:
         raise KernelError(f"silu_mul: input width {two_i} is odd")
     _need(out, "silu_mul out", gate_up.dtype, (n, two_i // 2))
     _check(_fn("core", "cpmcu_silu_mul")(_p(gate_up), _p(out), c_int(_code(out)), c_int(n), c_int(two_i // 2),
-                                         c_int(_act(activation)), _stream()))
+                                         *_act(activation), _stream()))
 
 
 def rope_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, hd: int, positions: torch.Tensor,
@@ -640,10 +652,11 @@ def rotate_copy(src: torch.Tensor, src_off: int, src_head_stride: int, heads: in
 def qkv_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, rot_dims: int,
                      positions: torch.Tensor, tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mag: float,
                      kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
-                     page_size: int, write_kv: bool = True):
+                     page_size: int, write_kv: bool = True, interleaved: bool = False):
     """rotate_copy three times in one launch: a row of qkv is [q: nh*dk | k: nkv*dk | v: nkv*dv]; q goes, rotated
     in its first rot_dims features, to q_out [n, nh*dk], k rotated into the key pages, v into the value pages
-    (pools whose heads may be padded to a multiple of 16 features)."""
+    (pools whose heads may be padded to a multiple of 16 features).  ``interleaved``: the rotation pairs
+    neighbouring features (2i, 2i + 1) instead of (i, i + rot_dims/2)."""
     ld = _ld(qkv, "qkv")
     n = qkv.shape[0]
     if qkv.shape[1] < nh * dk + (nkv * (dk + dv) if write_kv else 0):
@@ -665,7 +678,7 @@ def qkv_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, 
         _p(qkv), c_long(ld), c_int(_code(qkv)), _p(q_out), c_int(n), c_int(nh), c_int(nkv), c_int(dk), c_int(dv),
         c_int(rot_dims), _p(positions), _p(tok_slot), _p(inv_freq), c_float(mag), _p(kpool if write_kv else None),
         _p(vpool if write_kv else None), _p(page_table if write_kv else None), c_int(tw), c_int(page_size), c_int(pk),
-        c_int(pv), c_int(1 if write_kv else 0), _stream()))
+        c_int(pv), c_int(1 if write_kv else 0), c_int(1 if interleaved else 0), _stream()))
 
 
 def qkv_norm_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, rot_dims: int,
@@ -674,13 +687,14 @@ def qkv_norm_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: 
                           page_table: Optional[torch.Tensor], page_size: int, write_kv: bool = True,
                           bias: Optional[torch.Tensor] = None, q_norm: Optional[torch.Tensor] = None,
                           k_norm: Optional[torch.Tensor] = None, eps: float = 0.0, values_from_keys: bool = False,
-                          norm_after: bool = False):
+                          norm_after: bool = False, interleaved: bool = False):
     """qkv_rotate_store with what some designs put between projection and rotation: ``bias`` (float32, as wide as
     a row of qkv) is added; q heads and k heads are divided by their root mean square (eps inside the root) and
     multiplied by a weight of dk numbers shared by the heads (q_norm, k_norm, float32 [dk]); with
     values_from_keys a row is [q | k] only and the value pages receive k as projected (with its bias, before norm
     and rotation).  With norm_after the q and k heads are rotated first and then divided by their root mean square
-    (times q_norm / k_norm where given, by nothing else where not)."""
+    (times q_norm / k_norm where given, by nothing else where not).  ``interleaved`` as in qkv_rotate_store.  The
+    rows of qkv may be float32 where q_out and the cache are bfloat16 (rows that a convolution wrote)."""
     ld = _ld(qkv, "qkv")
     n = qkv.shape[0]
     width = nh * dk + ((nkv * dk + (0 if values_from_keys else nkv * dv)) if write_kv else 0)
@@ -688,7 +702,9 @@ def qkv_norm_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: 
         raise KernelError(f"qkv_norm_rotate_store: rows of {qkv.shape[1]} cannot hold {nh} query heads and {nkv} key/value heads")
     if values_from_keys and dv != dk:
         raise KernelError(f"qkv_norm_rotate_store: values that are the keys have the keys' size ({dv}, {dk})")
-    _need(q_out, "qkv q_out", qkv.dtype, (n, nh * dk))
+    _need(q_out, "qkv q_out", shape=(n, nh * dk))
+    if qkv.dtype != q_out.dtype and qkv.dtype != torch.float32:
+        raise KernelError(f"qkv_norm_rotate_store: rows of {qkv.dtype} for outputs of {q_out.dtype}")
     _need(positions, "qkv positions", torch.int32, (n,))
     if rot_dims:
         _need(inv_freq, "qkv inv_freq", torch.float32, (rot_dims // 2,))
@@ -703,17 +719,18 @@ def qkv_norm_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: 
     if write_kv:
         _need(tok_slot, "qkv token slots", torch.int32, (n,))
         _need(page_table, "qkv page table", torch.int32, (None, None))
-        _need(kpool, "qkv key pool", qkv.dtype, (None, page_size, None))
-        _need(vpool, "qkv value pool", qkv.dtype, (kpool.shape[0], page_size, None))
+        _need(kpool, "qkv key pool", q_out.dtype, (None, page_size, None))
+        _need(vpool, "qkv value pool", q_out.dtype, (kpool.shape[0], page_size, None))
         if kpool.shape[2] % nkv or vpool.shape[2] % nkv:
             raise KernelError(f"qkv_norm_rotate_store: pools of {kpool.shape[2]} / {vpool.shape[2]} features do not hold {nkv} heads")
         tw, pk, pv = page_table.shape[1], kpool.shape[2] // nkv, vpool.shape[2] // nkv
     _check(_fn("attention_general", "cpmcu_qkv_norm_rotate_store")(
-        _p(qkv), c_long(ld), c_int(_code(qkv)), _p(bias), _p(q_out), c_int(n), c_int(nh), c_int(nkv), c_int(dk), c_int(dv),
+        _p(qkv), c_long(ld), c_int(_code(q_out)), _p(bias), _p(q_out), c_int(n), c_int(nh), c_int(nkv), c_int(dk), c_int(dv),
         c_int(rot_dims), _p(q_norm), _p(k_norm), c_float(eps), c_int(1 if values_from_keys else 0), _p(positions),
         _p(tok_slot), _p(inv_freq), c_float(mag), _p(kpool if write_kv else None), _p(vpool if write_kv else None),
         _p(page_table if write_kv else None), c_int(tw), c_int(page_size), c_int(pk), c_int(pv),
-        c_int(1 if write_kv else 0), c_int(1 if norm_after else 0), _stream()))
+        c_int(1 if write_kv else 0), c_int(1 if norm_after else 0), c_int(1 if interleaved else 0), c_int(_code(qkv)),
+        _stream()))
 
 
 def _parts_of(t: torch.Tensor, n: int, H: int, name: str):
@@ -756,6 +773,51 @@ def bias_sum(a: torch.Tensor, bias: torch.Tensor, out: torch.Tensor):
     _need(bias, "bias", torch.float32, (H,))
     _check(_fn("norms", "cpmcu_bias_sum")(_p(a), c_int(_code(a)), c_int(parts), c_long(stride), _p(bias), _p(out),
                                           c_int(n), c_int(H), _stream()))
+
+
+def scaled_branches(a: torch.Tensor, a_bias: Optional[torch.Tensor], a_weight: Optional[torch.Tensor], a_scale: float,
+                    f: Optional[torch.Tensor], f_bias: Optional[torch.Tensor], f_weight: Optional[torch.Tensor],
+                    f_scale: float, out: torch.Tensor):
+    """out = a_scale * a_weight * (a + a_bias) + f_scale * f_weight * (f + f_bias) in float: a and f [n, H] or float
+    partial sums [P, n, H]; the weights (float32 [H], a number a column) and biases may be None, and so may f."""
+    _need(out, "scaled out", torch.float32, (None, None))
+    n, H = out.shape
+    ap, astr = _parts_of(a, n, H, "scaled branch")
+    fp, fstr = _parts_of(f, n, H, "scaled second branch") if f is not None else (0, 0)
+    for t, name in ((a_bias, "branch bias"), (f_bias, "second branch bias"), (a_weight, "branch weight"),
+                    (f_weight, "second branch weight")):
+        if t is not None:
+            _need(t, name, torch.float32, (H,))
+    _check(_fn("norms", "cpmcu_scaled_branches")(
+        _p(a), c_int(_code(a)), c_int(ap), c_long(astr), _p(a_bias), _p(a_weight), c_float(a_scale), _p(f),
+        c_int(_code(f) if f is not None else 0), c_int(fp), c_long(fstr), _p(f_bias), _p(f_weight), c_float(f_scale),
+        _p(out), c_int(n), c_int(H), _stream()))
+
+
+def bigram_add(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, tok_slot: torch.Tensor,
+               prev_state: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor, out: torch.Tensor, buckets: int,
+               mul_prev: int, mul_cur: int, remember: bool = True):
+    """out[r] += float(table[(prev * mul_prev + ids[r] * mul_cur) % buckets]); a token at position 0 reads row
+    ``buckets`` (the last of the table's buckets + 1 rows).  prev is the token before it in its sequence: the row
+    above in the packed batch, or, for the first row a sequence brings, prev_state[slot] (int32 [slots]).  With
+    ``remember`` every sequence's slot then holds the last token it brought."""
+    _need(table, "bigram table", shape=(buckets + 1, None))
+    H = table.shape[1]
+    _need(ids, "bigram ids", torch.int32, (None,))
+    n = ids.shape[0]
+    _need(positions, "bigram positions", torch.int32, (n,))
+    _need(tok_slot, "bigram token slots", torch.int32, (n,))
+    _need(prev_state, "bigram previous tokens", torch.int32, (None,))
+    _need(cu_q, "bigram sequence starts", torch.int32, (None,))
+    B = cu_q.shape[0] - 1
+    _need(seq_slot, "bigram sequence slots", torch.int32, (B,))
+    _need(out, "bigram out", torch.float32, (n, H))
+    if buckets <= 0 or mul_prev < 0 or mul_cur < 0:
+        raise KernelError(f"bigram_add: {buckets} buckets, multipliers {mul_prev}, {mul_cur}")
+    _check(_fn("core", "cpmcu_bigram_add")(_p(table), c_int(_code(table)), _p(ids), _p(positions), _p(tok_slot),
+                                           _p(prev_state), _p(cu_q), _p(seq_slot), _p(out), c_int(n), c_int(B), c_int(H),
+                                           c_long(buckets), c_long(mul_prev), c_long(mul_cur),
+                                           c_int(1 if remember else 0), _stream()))
 
 
 def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: int, f_off: int, i_bias: torch.Tensor,
@@ -880,33 +942,79 @@ def softcap(logits: torch.Tensor, cap: float):
     _check(_fn("core", "cpmcu_softcap")(_p(logits), c_long(logits.numel()), c_float(cap), _stream()))
 
 
-def delta_scan(qkv: torch.Tensor, gates: torch.Tensor, a_off: int, b_off: int, dt_bias: torch.Tensor,
+def delta_scan(qkv: torch.Tensor, gates: Optional[torch.Tensor], a_off: int, b_off: int, dt_bias: Optional[torch.Tensor],
                A_log: torch.Tensor, state: torch.Tensor, y: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor,
-               heads: int, kv_heads: int, dk: int, dv: int, q_scale: float, write_state: bool = True, lanes: int = 0):
+               heads: int, kv_heads: int, dk: int, dv: int, q_scale: float, write_state: bool = True, lanes: int = 0,
+               rule: str = "delta", channel_decay: Optional[torch.Tensor] = None):
     """The gated delta rule over each sequence's tokens, in float.  qkv float32 [n, 2*kv_heads*dk + heads*dv] =
     [q | k | v]; gates [n, W] holds the raw decay projection at columns a_off.. and the raw beta projection at
     b_off.. (heads each).  Per head (its q, k from head h // (heads/kv_heads)): q, k made unit vectors
     (x / sqrt(sum x^2 + 1e-6)), q times q_scale; beta = sigmoid(b); g = exp(-exp(A_log) softplus(a + dt_bias));
     S <- g S; u = beta (v - S^T k); S <- S + k u^T; y = S^T q.  state float32 [slots, heads, dv, dk]; y float32
     [n, heads*dv].  lanes: how many lanes share a column of the state (8 or 16; 0: chosen by how much the batch
-    gives the chip to do)."""
+    gives the chip to do).
+    rule 'channel': the decay is a number a head and key channel, S <- diag(g) S with g = exp(-exp(A_log[h])
+    softplus(channel_decay[:, h*dk + i] + dt_bias[h*dk + i])); channel_decay float32 [n, heads*dk] (may be a column
+    slice), dt_bias float32 [heads*dk]; a_off is not read.
+    rule 'decay': linear attention with a fixed decay a head, S <- A_log[h] S + k v^T, y = S^T q, q and k as they
+    come; no gates, no dt_bias (A_log holds the decays themselves)."""
+    if rule not in DELTA_RULES:
+        raise KernelError(f"delta_scan: rule '{rule}' ({sorted(DELTA_RULES)})")
     _need(qkv, "delta inputs", torch.float32, (None, 2 * kv_heads * dk + heads * dv))
     n = qkv.shape[0]
-    ldg = _ld(gates, "delta gates")
-    if gates.shape[0] != n or min(a_off, b_off) < 0 or max(a_off, b_off) + heads > gates.shape[1]:
-        raise KernelError(f"delta_scan: gate columns {a_off}, {b_off} (+{heads}) lie beyond rows of {tuple(gates.shape)}")
-    _need(dt_bias, "delta dt_bias", torch.float32, (heads,))
+    ldg = ld_a = 0
+    if rule != "decay":
+        ldg = _ld(gates, "delta gates")
+        cols = (b_off,) if rule == "channel" else (a_off, b_off)
+        if gates.shape[0] != n or min(cols) < 0 or max(cols) + heads > gates.shape[1]:
+            raise KernelError(f"delta_scan: gate columns {cols} (+{heads}) lie beyond rows of {tuple(gates.shape)}")
+        _need(dt_bias, "delta dt_bias", torch.float32, (heads * dk if rule == "channel" else heads,))
+    if rule == "channel":
+        ld_a = _ld(channel_decay, "delta channel decay")
+        if channel_decay.dtype != torch.float32 or tuple(channel_decay.shape) != (n, heads * dk):
+            raise KernelError(f"delta_scan: channel decay {channel_decay.dtype} {tuple(channel_decay.shape)}, expected "
+                              f"float32 {(n, heads * dk)}")
     _need(A_log, "delta A_log", torch.float32, (heads,))
     _need(state, "delta state", torch.float32, (None, heads, dv, dk))
     _need(y, "delta out", torch.float32, (n, heads * dv))
     _need(cu_q, "delta sequence starts", torch.int32, (None,))
     B = cu_q.shape[0] - 1
     _need(seq_slot, "delta sequence slots", torch.int32, (B,))
-    _check(_fn("delta", "cpmcu_delta_scan")(_p(qkv), c_long(qkv.shape[1]), _p(gates), c_long(ldg), c_int(_code(gates)),
-                                            c_long(a_off), c_long(b_off), _p(dt_bias), _p(A_log), _p(state), _p(y),
+    _check(_fn("delta", "cpmcu_delta_scan")(_p(qkv), c_long(qkv.shape[1]), _p(gates), c_long(ldg),
+                                            c_int(_code(gates) if gates is not None else 0), c_long(a_off), c_long(b_off),
+                                            _p(channel_decay), c_long(ld_a), _p(dt_bias), _p(A_log), _p(state), _p(y),
                                             _p(cu_q), _p(seq_slot), c_int(B), c_int(heads), c_int(kv_heads), c_int(dk),
                                             c_int(dv), c_float(q_scale), c_int(1 if write_state else 0), c_int(lanes),
-                                            _stream()))
+                                            c_int(DELTA_RULES[rule]), _stream()))
+
+
+DELTA_RULES = {"delta": 0, "channel": 1, "decay": 2}
+
+
+def linear_attention_prepare(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, out: torch.Tensor, heads: int,
+                             dk: int, dv: int, silu: bool, positions: Optional[torch.Tensor] = None,
+                             inv_freq: Optional[torch.Tensor] = None, interleaved: bool = False, k_scale: float = 1.0):
+    """What linear attention puts between its projection and its recurrence, in float: proj [n, W] holds q heads at
+    column q_off and k heads at k_off (heads x dk each) and v heads at v_off (heads x dv); out float32
+    [n, 2*heads*dk + heads*dv] = [q | k | v].  With silu all three pass z sigmoid(z); with inv_freq (float32
+    [r/2]) the first r features of q and k heads are rotated by positions * inv_freq (pairs (i, i + r/2), or
+    neighbours when interleaved); k is multiplied by k_scale."""
+    ld = _ld(proj, "linear attention projection")
+    n = proj.shape[0]
+    if min(q_off, k_off, v_off) < 0 or max(q_off + heads * dk, k_off + heads * dk, v_off + heads * dv) > proj.shape[1]:
+        raise KernelError(f"linear_attention_prepare: columns beyond rows of {tuple(proj.shape)}")
+    _need(out, "linear attention inputs", torch.float32, (n, 2 * heads * dk + heads * dv))
+    rot = 0
+    if inv_freq is not None:
+        _need(inv_freq, "linear attention inv_freq", torch.float32, (None,))
+        rot = 2 * inv_freq.shape[0]
+        _need(positions, "linear attention positions", torch.int32, (n,))
+        if rot > dk:
+            raise KernelError(f"linear_attention_prepare: the rotation covers {rot} features, a head has {dk}")
+    _check(_fn("delta", "cpmcu_linear_attention_prepare")(
+        _p(proj), c_int(_code(proj)), c_long(ld), c_long(q_off), c_long(k_off), c_long(v_off), _p(out), c_int(n),
+        c_int(heads), c_int(dk), c_int(dv), c_int(1 if silu else 0), c_int(rot), c_int(1 if interleaved else 0),
+        _p(inv_freq), _p(positions), c_float(k_scale), _stream()))
 
 
 def diff_qkv_store(src: torch.Tensor, q_out: torch.Tensor, heads: int, kv_heads: int, dk: int, dv: int,
@@ -953,15 +1061,20 @@ def diff_combine(a: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, 
 
 
 MOE_MAX_EXPERTS = 1024
+MOE_SCORES = {"softmax": 0, "sigmoid": 1}
+MOE_GROUP_SCORES = {"max": 0, "top2_sum": 1}
 
 
 def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor],
               n_groups: int, keep_groups: int, top: int, idx: torch.Tensor, weights: torch.Tensor,
-              shared_out: Optional[torch.Tensor] = None, logits: Optional[torch.Tensor] = None):
+              shared_out: Optional[torch.Tensor] = None, logits: Optional[torch.Tensor] = None,
+              score: str = "softmax", group_score: str = "max", weight_scale: float = 1.0):
     """Routing of every token to ``top`` of E experts.  Logits router . h in float (router float32 [E, H]), scores
-    s = softmax; choice scores s + correction; the experts form n_groups equal groups of neighbours, of which only
-    the keep_groups with the largest best choice score may be chosen from; the top largest choice scores win (ties:
-    the lower index); weights = s of the chosen / (their sum + 1e-20).  idx int32 [n, top], weights float32 [n, top].
+    s = softmax over the experts (``score`` 'sigmoid': of each logit alone); choice scores s + correction; the
+    experts form n_groups equal groups of neighbours, of which only the keep_groups with the largest group score may
+    be chosen from (``group_score`` 'max': a group's best choice score; 'top2_sum': the sum of its two best); the top
+    largest choice scores win (ties: the lower index); weights = s of the chosen / (their sum + 1e-20) *
+    weight_scale.  idx int32 [n, top], weights float32 [n, top].
     shared_gate (float32 [H]): shared_out[t] = sigmoid(shared_gate . h[t]).  logits: float32 [n, E + 1] of scratch
     (allocated here when absent: a caller that must not allocate brings it)."""
     ldh = _ld(h, "router input")
@@ -978,14 +1091,18 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.
     if logits is None:
         logits = torch.empty((n, E + 1), dtype=torch.float32, device=h.device)
     _need(logits, "router logits", torch.float32, (n, E + 1))
+    if score not in MOE_SCORES or group_score not in MOE_GROUP_SCORES:
+        raise KernelError(f"moe_route: score '{score}' ({sorted(MOE_SCORES)}) or group score '{group_score}' "
+                          f"({sorted(MOE_GROUP_SCORES)}) is not known")
     _check(_fn("moe", "cpmcu_moe_route")(_p(h), c_long(ldh), c_int(_code(h)), _p(router), _p(correction), _p(shared_gate),
                                          c_int(n), c_int(H), c_int(E), c_int(n_groups), c_int(keep_groups), c_int(top),
-                                         _p(logits), _p(idx), _p(weights), _p(shared_out), _stream()))
+                                         _p(logits), _p(idx), _p(weights), _p(shared_out), c_int(MOE_SCORES[score]),
+                                         c_int(MOE_GROUP_SCORES[group_score]), c_float(weight_scale), _stream()))
 
 
-def moe_gated(h: torch.Tensor, gate_up: torch.Tensor, idx: torch.Tensor, act: torch.Tensor):
-    """act[t, k] = silu(Wg_e h[t]) * (Wu_e h[t]) for e = idx[t, k]; gate_up [E, 2F, H] (an expert's gate rows, then
-    its up rows), act [n, top, F], both of h's element type."""
+def moe_gated(h: torch.Tensor, gate_up: torch.Tensor, idx: torch.Tensor, act: torch.Tensor, activation="silu"):
+    """act[t, k] = act(Wg_e h[t]) * (Wu_e h[t]) for e = idx[t, k] (act: SiLU, or as gate_activation says); gate_up
+    [E, 2F, H] (an expert's gate rows, then its up rows), act [n, top, F], both of h's element type."""
     ldh = _ld(h, "experts input")
     n, H = h.shape
     _need(gate_up, "experts gate/up", h.dtype, (None, None, H))
@@ -996,7 +1113,7 @@ def moe_gated(h: torch.Tensor, gate_up: torch.Tensor, idx: torch.Tensor, act: to
     top = idx.shape[1]
     _need(act, "experts act", h.dtype, (n, top, F2 // 2))
     _check(_fn("moe", "cpmcu_moe_gated")(_p(h), c_long(ldh), c_int(_code(h)), _p(gate_up), _p(idx), _p(act), c_int(n),
-                                         c_int(H), c_int(F2 // 2), c_int(top), _stream()))
+                                         c_int(H), c_int(F2 // 2), c_int(top), *_act(activation), _stream()))
 
 
 def moe_down(act: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, weights: torch.Tensor, out: torch.Tensor,
@@ -1035,7 +1152,7 @@ def moe_experts_mfma_ok(h: torch.Tensor, expert_size: int, n_tiles: int) -> bool
 def moe_experts_mfma(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, weights: torch.Tensor,
                      out: torch.Tensor, act: torch.Tensor, y: torch.Tensor, rows: torch.Tensor, tile_expert: torch.Tensor,
                      n_tiles: torch.Tensor, shared: Optional[torch.Tensor] = None,
-                     shared_gate: Optional[torch.Tensor] = None):
+                     shared_gate: Optional[torch.Tensor] = None, activation="silu"):
     """moe_gated + moe_down for steps of many tokens, bf16 on the matrix cores: the (token, expert) pairs are grouped
     by expert into tiles of MOE_TILE rows.  Scratch: act bf16 [n, top, F], y bf16 [n, top, H], rows int32
     [tiles * MOE_TILE], tile_expert int32 [tiles], n_tiles int32 [1], tiles >= moe_tiles(n, top, E)."""
@@ -1063,7 +1180,7 @@ def moe_experts_mfma(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
         _p(h), c_long(ldh), _p(gate_up), _p(down), _p(idx), _p(weights), _p(shared),
         c_int(_code(shared) if shared is not None else 0), c_int(sp), c_long(sstr), _p(shared_gate), _p(act), _p(y),
         _p(rows), _p(tile_expert), _p(n_tiles), c_int(tiles), _p(out), c_int(n), c_int(H), c_int(F), c_int(E), c_int(top),
-        _stream()))
+        *_act(activation), _stream()))
 
 
 def latent_store(proj: torch.Tensor, q_out: torch.Tensor, nh: int, dim: int, rot: int, rank: int,
@@ -1108,8 +1225,10 @@ def _value_heads(nkv: int, v_share: int) -> int:
 def attention_general(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk: int, hdv: int, scale: float,
                       kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
                       positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0, window: int = 0,
-                      keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1):
+                      keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1,
+                      softcap: float = 0.0):
     """Causal attention with key size hdk and value size hdv of their own (plain kernel, both element types).
+    softcap c > 0: a scaled score s enters the softmax as c tanh(s / c).
     v_share: runs of that many neighbouring key heads read one value head (the value pool holds nkv / v_share heads).
     The cache may hold heads padded to a multiple of 16 features.  chunk > 0: the query at position p sees only
     keys j <= p with j // chunk == p // chunk.  window > 0: only keys with p - j < window, and the sequence's
@@ -1133,7 +1252,7 @@ def attention_general(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk
         c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nvh), c_float(scale), c_int(chunk), c_int(window),
         c_int(keep_first), _p(sink), _p(kpool),
         _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
-        c_int(v_share), _stream()))
+        c_int(v_share), c_float(softcap or 0.0), _stream()))
 
 
 def gemm_heads(x: torch.Tensor, x_off: int, x_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_off: int,
@@ -1332,7 +1451,7 @@ def proj_add_norm(a: torch.Tensor, w: "TiledWeight", alpha: float, x: torch.Tens
 
 
 def gated_strip(x: torch.Tensor, w: "TiledWeight", out: torch.Tensor, row_scale: Optional[RowScale] = None,
-                activation: str = "silu"):
+                activation="silu"):
     """out = act(x . Wg^T) * (x . Wu^T) (act as in silu_mul) for a step of at most 16 tokens, w tiled with the gate rows first (a
     multiple of 16 of them); out bfloat16 [n, N/2].  With row_scale as in gemm_skinny."""
     _need(x, "gated x", torch.bfloat16, (None, None))
@@ -1346,11 +1465,11 @@ def gated_strip(x: torch.Tensor, w: "TiledWeight", out: torch.Tensor, row_scale:
                                            _p(row_scale.sums if row_scale is not None else None),
                                            c_int(row_scale.sums.shape[1] if row_scale is not None else 0),
                                            c_float(row_scale.eps if row_scale is not None else 0.0),
-                                           c_int(_act(activation)), _stream()))
+                                           *_act(activation), _stream()))
 
 
 def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain",
-                row_scale: Optional[RowScale] = None, activation: str = "silu"):
+                row_scale: Optional[RowScale] = None, activation="silu"):
     """bf16 product for at most 64 rows of x on the matrix cores, streaming w once; w is [N, K] as in the
     checkpoint or a TiledWeight.
     mode 'plain': out [m,N] float32 or bfloat16; 'partial': out float32 [S,m,N], S slices of K to be summed by
@@ -1387,7 +1506,7 @@ def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode:
                                             _p(row_scale.sums if row_scale is not None else None),
                                             c_int(row_scale.sums.shape[1] if row_scale is not None else 0),
                                             c_float(row_scale.eps if row_scale is not None else 0.0),
-                                            c_int(_act(activation)), _stream()))
+                                            *_act(activation), _stream()))
 
 
 SKINNY_MAX_ROWS = 64
@@ -1502,7 +1621,7 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
                            part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                            tiles: Optional[torch.Tensor] = None, tokens_per_tile: int = 1, window: int = 0,
                            keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1,
-                           gate: Optional[torch.Tensor] = None):
+                           gate: Optional[torch.Tensor] = None, softcap: float = 0.0):
     """attention_general in bf16 on the matrix cores (key size a multiple of 8 up to 1024, value size up to 512).
     With n_splits > 1 every token's visible keys are shared among n_splits workgroups and merged afterwards;
     part_o float32 [n, nh, n_splits, hdv] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
@@ -1543,7 +1662,7 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
         c_int(keep_first), _p(sink), _p(kpool), _p(vpool),
         _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot), c_int(n_splits),
         _p(tiles), c_int(tiles.shape[0] if tiles is not None else 0), c_int(tokens_per_tile), c_int(v_share),
-        _p(gate), c_long(ld_gate), _stream()))
+        _p(gate), c_long(ld_gate), c_float(softcap or 0.0), _stream()))
 
 
 def attention_general_tokens_per_tile(n_tokens: int, nh: int, nkv: int, pool_hdv: int) -> int:
@@ -1570,15 +1689,15 @@ def reserve_attention_general(ws, dtype, nh: int, nkv: int, hdv: int, pool_hdv: 
 
 def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx, chunk: int = 0,
                   window: int = 0, keep_first: int = 0, sink: Optional[torch.Tensor] = None, v_share: int = 1,
-                  gate: Optional[torch.Tensor] = None) -> bool:
+                  gate: Optional[torch.Tensor] = None, softcap: float = 0.0) -> bool:
     """Attention with key and value sizes of their own and an optional mask (chunks, or a sliding window with kept
     first tokens) and softmax sink, with the kernel that suits the step; writes ``out`` [n, nh*hdv] (q's type, or
     float32).  v_share: runs of that many neighbouring key heads read one value head.  gate [n, nh*hdv]: an output
     gate that the matrix-core kernel applies as it writes (out * sigmoid(gate)); returns whether it did, so that
-    the caller applies it itself after the other kernels."""
+    the caller applies it itself after the other kernels.  softcap c > 0: scaled scores pass c tanh(s / c)."""
     pool_hdv = vpool.shape[2] // _value_heads(nkv, v_share)
     if (hdk == hdv and chunk == 0 and window == 0 and sink is None and hdk <= 256 and hdk % 16 == 0
-            and kpool.shape[2] == nkv * hdk and v_share == 1):
+            and kpool.shape[2] == nkv * hdk and v_share == 1 and not softcap):
         attention(q, out, nh, nkv, hdk, scale, kpool, vpool, page_table, page_size, ctx)
         return False
     if attention_general_mfma_ok(q, hdk, hdv, page_size):
@@ -1603,15 +1722,15 @@ def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, pa
                     tiles = ctx.extras[key] = prefill_tiles(ctx.q_lens, tpt, q.device)
         attention_general_mfma(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
                                ctx.tok_slot, chunk, splits, part_o, part_ml, tiles, tpt, window, keep_first, sink, v_share,
-                               gate)
+                               gate, softcap)
         return gate is not None
     if out.dtype != q.dtype:
         # the plain kernel writes the type it reads: through scratch of that type
         tmp = ctx.ws.get("attn.gout_plain", tuple(out.shape), q.dtype)
         attention_general(q, tmp, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
-                          ctx.tok_slot, chunk, window, keep_first, sink, v_share)
+                          ctx.tok_slot, chunk, window, keep_first, sink, v_share, softcap)
         out.copy_(tmp)
         return False
     attention_general(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
-                      ctx.tok_slot, chunk, window, keep_first, sink, v_share)
+                      ctx.tok_slot, chunk, window, keep_first, sink, v_share, softcap)
     return False

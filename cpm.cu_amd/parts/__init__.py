@@ -11,6 +11,7 @@ from .mlstm import MLSTMMixer
 from .diff_attention import DifferentialAttention
 from .delta import GatedDeltaMixer
 from .parallel import ParallelMixer
+from .linear_attention import DecayLinearAttention
 from .ffn import GatedFFN, PolyNormFFN, RoutedExpertsFFN
-from .block import HyperConnectionBlock, ParallelGatedBlock, PreNormBlock, SandwichNormBlock
+from .block import HyperConnectionBlock, ParallelGatedBlock, ParallelScaledBlock, PreNormBlock, SandwichNormBlock
 from .embedding import LMHead, TokenEmbedding

@@ -22,7 +22,7 @@ from typing import List, Mapping, Optional
 import torch
 
 from .. import ops
-from ..cache.paged import CacheNeeds, CacheView, StreamSpec
+from ..cache.paged import CacheNeeds, CacheView, StateSpec, StreamSpec
 from .base import MIXERS, BiasedBranch, DeferredBranch, Mixer, Part, PositionEncoding, Runtime, StepContext
 from .linear import Linear
 
@@ -239,15 +239,22 @@ class GeneralAttention(Mixer):
                            no value and no scale;
       'gate'               an output gate: the heads side by side are multiplied element by element with
                            sigmoid(W_gate h) before the output projection (its rows ride in the q/k/v product).
+      'q_conv', 'k_conv', 'v_conv'   with ``conv_taps`` > 0: a short causal convolution over time on every channel of
+                           q, k and v ([channels, taps], the last tap the current token's, zeros before the start,
+                           no bias, no activation) directly behind the projection; the last taps - 1 projected rows
+                           of a sequence are fixed-size state of its cache slot.
     ``unit_norm_after_rotation``: q and k heads are divided by their root mean square (``norm_eps`` inside the
     root, no weight) after the rotation.
+    ``rotation_pairs``: 'halves' pairs feature i with i + r/2 of the r rotated features, 'interleaved' 2i with 2i + 1.
+    ``score_softcap`` c: a scaled score s enters the softmax as c tanh(s / c).
     Without 'v' the values are the keys as projected (with their bias, before norm and rotation): value_dim
     must equal key_dim."""
 
     def __init__(self, names: Mapping[str, str], hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int,
                  value_dim: int, position: Optional[PositionEncoding], scale: float, mask_chunk: Optional[int] = None,
                  mask_window: Optional[int] = None, mask_keep_first: int = 0, norm_eps: float = 0.0,
-                 unit_norm_after_rotation: bool = False):
+                 unit_norm_after_rotation: bool = False, rotation_pairs: str = "halves",
+                 score_softcap: Optional[float] = None, conv_taps: int = 0):
         if num_heads % num_kv_heads:
             raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         if unit_norm_after_rotation and (names.get("q_norm") or names.get("k_norm")):
@@ -262,8 +269,19 @@ class GeneralAttention(Mixer):
             raise ValueError("attention: a chunked mask or a sliding window, not both")
         if mask_keep_first < 0 or (mask_keep_first and not mask_window):
             raise ValueError("attention: kept first tokens come with a sliding window")
+        if rotation_pairs not in ("halves", "interleaved"):
+            raise ValueError(f"attention: rotation pairs '{rotation_pairs}' (halves or interleaved)")
+        if score_softcap is not None and not score_softcap > 0:
+            raise ValueError(f"attention: a score cap of {score_softcap}")
+        if conv_taps < 0:
+            raise ValueError(f"attention: {conv_taps} convolution taps")
+        self.interleaved = rotation_pairs == "interleaved"
+        self.softcap = float(score_softcap) if score_softcap is not None else 0.0
+        self.taps = int(conv_taps)
         self.names = dict(names)
         self.values_are_keys = "v" not in self.names
+        if self.taps and (self.values_are_keys or self.names.get("gate")):
+            raise ValueError("attention: the convolution goes with q, k and v of their own and no output gate")
         if self.values_are_keys and value_dim != key_dim:
             raise ValueError(f"attention: values that are the keys have the keys' size ({value_dim}, {key_dim})")
         self.hidden_size, self.nh, self.nkv, self.dk, self.dv = hidden_size, num_heads, num_kv_heads, key_dim, value_dim
@@ -285,7 +303,8 @@ class GeneralAttention(Mixer):
                         bias_names=[self.names["out_bias"]] if self.names.get("out_bias") else None)
         # what the plain rotate-and-store kernel does not do
         self._extras = bool(any(biases) or self.names.get("q_norm") or self.names.get("k_norm") or self.values_are_keys
-                            or self.norm_after)
+                            or self.norm_after or self.taps)
+        self.conv_widths = (num_heads * key_dim, num_kv_heads * key_dim, num_kv_heads * value_dim)
 
     def parts(self) -> List[Part]:
         return [self.qkv, self.o] + ([self.position] if self.position is not None else [])
@@ -295,16 +314,24 @@ class GeneralAttention(Mixer):
         specs = [WeightSpec(self.names[k], (self.dk,), "norm") for k in ("q_norm", "k_norm") if self.names.get(k)]
         if self.names.get("sink"):
             specs.append(WeightSpec(self.names["sink"], (self.nh,), "small"))
+        if self.taps:
+            specs += [WeightSpec(self.names[k], (w, self.taps), "conv_taps")
+                      for k, w in zip(("q_conv", "k_conv", "v_conv"), self.conv_widths)]
         return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
         self.rt = rt
         f = lambda k: tensors[self.names[k]].to(torch.float32).contiguous() if self.names.get(k) else None
         self.q_norm, self.k_norm, self.sink = f("q_norm"), f("k_norm"), f("sink")
+        if self.taps:
+            self.conv_w = torch.cat([f("q_conv"), f("k_conv"), f("v_conv")], 0).contiguous()
 
     def cache_needs(self) -> CacheNeeds:
+        state = ()
+        if self.taps > 1:
+            state = (("conv", StateSpec((self.taps - 1, sum(self.conv_widths)), torch.float32)),)
         return CacheNeeds(streams=(("k", StreamSpec(self.nkv * _pad16(self.dk))),
-                                   ("v", StreamSpec(self.nkv * _pad16(self.dv)))),
+                                   ("v", StreamSpec(self.nkv * _pad16(self.dv)))), state=state,
                           window=self.chunk or self.window or None, keep_first=self.keep_first)
 
     def reserve_workspace(self, ws, rt: Runtime, max_step_tokens: int, max_slots: int):
@@ -324,26 +351,34 @@ class GeneralAttention(Mixer):
         rd = 0 if inv_freq is None else 2 * inv_freq.shape[0]
         if rd > dk:
             raise ValueError(f"attention: the rotation covers {rd} features, a head has {dk}")
+        if self.taps and not writes_cache:
+            raise ValueError("attention: a run that reads another run's cache has no convolution state of its own")
         with ctx.timed("attn_qkv_rope"):
             qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if (writes_cache or self.gate_off is not None) else nh * dk)
+            if self.taps:
+                # the projected rows mixed over time, in float; the slot's state moves on to the step's last rows
+                mixed = ctx.ws.get("attn.conv", (n, sum(self.conv_widths)), torch.float32)
+                ops.conv_silu(qkv, self.conv_w, None, cache.state.get("conv"), mixed, ctx.cu_q, ctx.seq_slot,
+                              max(ctx.q_lens), update_state=True, activation=False)
+                qkv = mixed
             q = ctx.ws.get("attn.q", (n, nh * dk), self.rt.dtype)
             if self._extras:
                 ops.qkv_norm_rotate_store(qkv, q, nh, nkv, dk, dv, rd, ctx.positions, ctx.tok_slot, inv_freq, mag,
                                           cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
                                           write_kv=writes_cache, bias=self.qkv.bias, q_norm=self.q_norm,
                                           k_norm=self.k_norm, eps=self.norm_eps, values_from_keys=self.values_are_keys,
-                                          norm_after=self.norm_after)
+                                          norm_after=self.norm_after, interleaved=self.interleaved)
             else:
                 ops.qkv_rotate_store(qkv, q, nh, nkv, dk, dv, rd, ctx.positions, ctx.tok_slot, inv_freq, mag,
                                      cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
-                                     write_kv=writes_cache)
+                                     write_kv=writes_cache, interleaved=self.interleaved)
         out = ctx.ws.get("attn.out", (n, nh * dv), self.rt.dtype)
         gate = qkv[:, self.gate_off:self.gate_off + nh * dv] if self.gate_off is not None else None
         with ctx.timed("attn_core"):
             # the matrix-core kernel (and the merge of split keys) applies the gate as it writes
             gated_there = ops.attention_any(q, out, nh, nkv, dk, dv, self.scale, cache.streams["k"], cache.streams["v"],
                                             cache.page_table, cache.page_size, ctx, chunk=self.chunk, window=self.window,
-                                            keep_first=self.keep_first, sink=self.sink, gate=gate)
+                                            keep_first=self.keep_first, sink=self.sink, gate=gate, softcap=self.softcap)
         if gate is not None and not gated_there:
             with ctx.timed("attn_gate"):
                 gated = ctx.ws.get("attn.gated", (n, nh * dv), self.rt.dtype)

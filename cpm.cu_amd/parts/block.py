@@ -166,6 +166,56 @@ class ParallelGatedBlock(Block):
         stream.pending_scale = 1.0
 
 
+@BLOCKS.register("parallel_scaled")
+class ParallelScaledBlock(Block):
+    """One norm a layer, both sub-layers read its output, and each sub-layer's result is multiplied element by
+    element by a learned vector (a layer scale) before the two join the residual: with h = norm(x),
+
+        x += s1 * Mixer(h) + s2 * FeedForward(h)
+
+    A layer may have no feed-forward (the second term and its vector are then absent).  The sum is left pending
+    (float) for the norm that follows.  ``scale_names``: checkpoint tensors of s1 and, with a feed-forward, s2."""
+
+    def __init__(self, norm: Norm, mixer: Mixer, feed_forward: Optional[FeedForward], hidden_size: int,
+                 scale_names: List[str]):
+        if len(scale_names) != (2 if feed_forward is not None else 1):
+            raise ValueError("parallel_scaled: one scale vector for every sub-layer")
+        self.norm, self.mixer, self.feed_forward, self.hidden_size = norm, mixer, feed_forward, hidden_size
+        self.scale_names = list(scale_names)
+
+    def parts(self) -> List[Part]:
+        return [self.norm, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else [])
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return [WeightSpec(name, (self.hidden_size,), "norm") for name in self.scale_names]
+
+    def bind(self, tensors, rt: Runtime):
+        self.scales = [tensors[name].to(torch.float32).contiguous() for name in self.scale_names]
+
+    @staticmethod
+    def _with_bias(branch):
+        if isinstance(branch, BiasedBranch):
+            return branch.branch, branch.bias
+        return branch_tensor(branch), None
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True):
+        with ctx.timed("norm"):
+            h = self.norm.forward(stream.x, branch_for(self.norm, stream.take_pending()), stream.pending_scale, ctx,
+                                  tag="block.h")
+        with ctx.timed("attn"):
+            a, a_bias = self._with_bias(self.mixer.forward(h, ctx, cache, writes_cache))
+        f = f_bias = None
+        if self.feed_forward is not None:
+            with ctx.timed("ffn"):
+                f, f_bias = self._with_bias(self.feed_forward.forward(h, ctx))
+        with ctx.timed("layer_scale"):
+            out = ctx.ws.get("block.scaled", (h.shape[0], self.hidden_size), torch.float32)
+            ops.scaled_branches(a, a_bias, self.scales[0], 1.0, f, f_bias, self.scales[1] if f is not None else None, 1.0,
+                                out)
+        stream.pending = out
+        stream.pending_scale = 1.0
+
+
 @BLOCKS.register("hyper_connections")
 class HyperConnectionBlock(Block):
     """Pre-norm sub-layers over a residual of S streams (hyper-connections).  Sub-layer q (1: mixer, 2:

@@ -1,4 +1,4 @@
-"""Gated feed-forward: down( act(x Wg^T) * (x Wu^T) ), act = SiLU (or the tanh form of GELU).
+"""Gated feed-forward: down( act(x Wg^T) * (x Wu^T) ), act = SiLU (or the tanh form of GELU, or a clamped swish).
 
 gate and up are one stacked product, gate rows first (src/model/ffn.cuh:31-59,
 77-84); silu(g) * u in float (src/model/activation.cuh:6-18).
@@ -18,13 +18,16 @@ from .linear import Linear
 @FEED_FORWARDS.register("gated_silu")
 class GatedFFN(FeedForward):
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, names: Optional[Mapping[str, str]] = None,
-                 activation: str = "silu"):
+                 activation="silu"):
         """``names``: the checkpoint tensors for 'gate', 'up', 'down' behind the prefix (default: the MiniCPM
         checkpoint's gate_proj.weight, up_proj.weight, down_proj.weight).  ``activation``: the gate's
-        nonlinearity, 'silu' or 'gelu_tanh' (0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))))."""
-        if activation not in ops.GATE_ACTIVATIONS:
-            raise ValueError(f"feed-forward: gate nonlinearity '{activation}' (known: {sorted(ops.GATE_ACTIVATIONS)})")
-        self.activation = activation
+        nonlinearity, 'silu' or 'gelu_tanh' (0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))), or
+        ('clamped_swish', limit): g <- min(g, limit), up <- clamp(up, -limit, limit), and the pair's product is
+        g sigmoid(1.702 g) (up + 1)."""
+        try:
+            self.activation = ops.gate_activation(activation)
+        except ops.KernelError as e:
+            raise ValueError(f"feed-forward: {e}") from None
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         names = names or {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
@@ -86,20 +89,23 @@ class PolyNormFFN(FeedForward):
 
 @FEED_FORWARDS.register("routed_experts")
 class RoutedExpertsFFN(FeedForward):
-    """A mixture of small SiLU-gated feed-forwards (no biases), of which every token uses ``top``.
+    """A mixture of small gated feed-forwards (no biases), of which every token uses ``top``.
 
-    Router: logits z = W_router h in float, scores s = softmax(z) over all experts.  The choice goes by s + a
-    correction a expert (a checkpoint tensor; the weights use s without it).  With ``groups`` = (count, keep) the
-    experts form ``count`` equal groups of neighbours, a group's score is its largest choice score, and only experts
-    of the ``keep`` best groups can be chosen.  The chosen experts' outputs are added with weights s / (sum of the
-    chosen s + 1e-20).  A shared expert (``shared_size``) runs for every token and is added times sigmoid(w . h),
-    one number a token.
+    Router: logits z = W_router h in float, scores s = softmax(z) over all experts (``score`` 'sigmoid': sigmoid of
+    every logit alone).  The choice goes by s + a correction a expert (a checkpoint tensor; the weights use s without
+    it).  With ``groups`` = (count, keep) the experts form ``count`` equal groups of neighbours, a group's score is
+    its largest choice score (``group_score`` 'top2_sum': the sum of its two largest), and only experts of the
+    ``keep`` best groups can be chosen.  The chosen experts' outputs are added with weights s / (sum of the chosen s +
+    1e-20) * ``weight_scale``.  A shared expert (``shared_size``) runs for every token and is added, times
+    sigmoid(w . h), one number a token, if ``names`` holds 'shared_scale'.  ``activation`` / ``shared_activation``:
+    the experts' and the shared expert's nonlinearity as GatedFFN takes it.
 
     ``names``: 'router', 'correction' (or absent), 'expert' (a format with {e} for the expert's number and {part}
     for gate / up / down), and for the shared expert 'shared_gate', 'shared_up', 'shared_down', 'shared_scale'."""
 
     def __init__(self, names: Mapping[str, str], hidden_size: int, expert_size: int, experts: int, top: int,
-                 groups: Optional[Tuple[int, int]] = None, shared_size: Optional[int] = None):
+                 groups: Optional[Tuple[int, int]] = None, shared_size: Optional[int] = None, score: str = "softmax",
+                 group_score: str = "max", weight_scale: float = 1.0, activation="silu", shared_activation=None):
         if experts > ops.MOE_MAX_EXPERTS:
             raise ValueError(f"routed_experts: {experts} experts (up to {ops.MOE_MAX_EXPERTS} are taken)")
         if not 0 < top <= experts:
@@ -108,6 +114,14 @@ class RoutedExpertsFFN(FeedForward):
             count, keep = groups
             if count <= 0 or experts % count or not 0 < keep <= count or top > keep * (experts // count):
                 raise ValueError(f"routed_experts: {experts} experts in {count} groups, {keep} kept, {top} chosen")
+        if score not in ops.MOE_SCORES or group_score not in ops.MOE_GROUP_SCORES:
+            raise ValueError(f"routed_experts: score '{score}' ({sorted(ops.MOE_SCORES)}) or group score "
+                             f"'{group_score}' ({sorted(ops.MOE_GROUP_SCORES)})")
+        try:
+            self.activation = ops.gate_activation(activation)
+        except ops.KernelError as e:
+            raise ValueError(f"routed_experts: {e}") from None
+        self.score, self.group_score, self.weight_scale = score, group_score, float(weight_scale)
         self.names = dict(names)
         self.hidden_size, self.expert_size, self.experts, self.top = hidden_size, expert_size, experts, top
         self.groups = tuple(groups) if groups is not None else (1, 1)
@@ -115,7 +129,9 @@ class RoutedExpertsFFN(FeedForward):
         if shared_size is not None:
             self.shared = GatedFFN("", hidden_size, shared_size, names={"gate": self.names["shared_gate"],
                                                                         "up": self.names["shared_up"],
-                                                                        "down": self.names["shared_down"]})
+                                                                        "down": self.names["shared_down"]},
+                                   activation=shared_activation if shared_activation is not None else activation)
+        self.shared_gated = self.shared is not None and bool(self.names.get("shared_scale"))
 
     def _expert(self, e: int, part: str) -> str:
         return self.names["expert"].format(e=e, part=part)
@@ -131,7 +147,7 @@ class RoutedExpertsFFN(FeedForward):
         for e in range(self.experts):
             specs += [WeightSpec(self._expert(e, "gate"), (F, H)), WeightSpec(self._expert(e, "up"), (F, H)),
                       WeightSpec(self._expert(e, "down"), (H, F))]
-        if self.shared is not None:
+        if self.shared_gated:
             specs.append(WeightSpec(self.names["shared_scale"], (1, H)))
         return specs
 
@@ -140,7 +156,7 @@ class RoutedExpertsFFN(FeedForward):
         f32 = lambda name: tensors[name].to(torch.float32).contiguous()
         self.router = f32(self.names["router"])
         self.correction = f32(self.names["correction"]) if self.names.get("correction") else None
-        self.shared_scale = f32(self.names["shared_scale"]).reshape(-1) if self.shared is not None else None
+        self.shared_scale = f32(self.names["shared_scale"]).reshape(-1) if self.shared_gated else None
         # an expert's gate rows, then its up rows: [E, 2F, H]; down: [E, H, F]
         self.gate_up = torch.stack([torch.cat([tensors[self._expert(e, "gate")], tensors[self._expert(e, "up")]], 0)
                                     for e in range(self.experts)]).to(rt.dtype).contiguous()
@@ -150,11 +166,12 @@ class RoutedExpertsFFN(FeedForward):
         n = h.shape[0]
         idx = ctx.ws.get("moe.idx", (n, self.top), torch.int32)
         wts = ctx.ws.get("moe.weights", (n, self.top), torch.float32)
-        sg = ctx.ws.get("moe.shared_gate", (n,), torch.float32) if self.shared is not None else None
+        sg = ctx.ws.get("moe.shared_gate", (n,), torch.float32) if self.shared_gated else None
         logits = ctx.ws.get("moe.logits", (n, self.experts + 1), torch.float32)
         with ctx.timed("moe_route"):
             ops.moe_route(h, self.router, self.correction, self.shared_scale, self.groups[0], self.groups[1], self.top,
-                          idx, wts, sg, logits)
+                          idx, wts, sg, logits, score=self.score, group_score=self.group_score,
+                          weight_scale=self.weight_scale)
         shared = self.shared.forward(h, ctx) if self.shared is not None else None
         act = ctx.ws.get("moe.act", (n, self.top, self.expert_size), self.rt.dtype)
         out = ctx.ws.get("moe.out", (n, self.hidden_size), torch.float32)
@@ -167,9 +184,9 @@ class RoutedExpertsFFN(FeedForward):
                 tile_expert = ctx.ws.get("moe.tile_expert", (tiles,), torch.int32)
                 n_tiles = ctx.ws.get("moe.n_tiles", (1,), torch.int32)
                 ops.moe_experts_mfma(h, self.gate_up, self.down, idx, wts, out, act, y, rows, tile_expert, n_tiles,
-                                     shared, sg)
+                                     shared, sg, activation=self.activation)
             else:
                 # few tokens: an expert's weights stream once for every token that chose it
-                ops.moe_gated(h, self.gate_up, idx, act)
+                ops.moe_gated(h, self.gate_up, idx, act, activation=self.activation)
                 ops.moe_down(act, self.down, idx, wts, out, shared, sg)
         return out

@@ -3,6 +3,8 @@ first divided by its root mean square over the model width and multiplied by a w
 
     y = (left(h) / rms(left(h)) * w_left + right(h) / rms(right(h)) * w_right) / 2
 
+or, with ``scales`` = (a, b) instead of the two norm weights, their plain weighted sum y = a left(h) + b right(h).
+
 The pair owns one cache entry; what the two mixers need of it (per-token streams, fixed-size state, a window) is put
 together under the prefixes ``left.`` and ``right.``, and each mixer sees its own part under its own names.
 """
@@ -19,9 +21,13 @@ from .base import MIXERS, BiasedBranch, Mixer, Part, Runtime, StepContext, Weigh
 
 @MIXERS.register("parallel")
 class ParallelMixer(Mixer):
-    def __init__(self, left: Mixer, right: Mixer, left_norm_name: str, right_norm_name: str, hidden_size: int, eps: float):
+    def __init__(self, left: Mixer, right: Mixer, left_norm_name: Optional[str] = None, right_norm_name: Optional[str] = None,
+                 hidden_size: int = 0, eps: float = 0.0, scales: Optional[tuple] = None):
+        if (scales is None) == (left_norm_name is None) or (left_norm_name is None) != (right_norm_name is None):
+            raise ValueError("parallel: either the two norm weights' names or the two numbers of a weighted sum")
         self.left, self.right = left, right
-        self.norm_names = (left_norm_name, right_norm_name)
+        self.norm_names = (left_norm_name, right_norm_name) if scales is None else ()
+        self.scales = (float(scales[0]), float(scales[1])) if scales is not None else None
         self.hidden_size, self.eps = hidden_size, float(eps)
         a, b = left.cache_needs(), right.cache_needs()
         if a.streams and b.streams and (a.window, a.keep_first) != (b.window, b.keep_first):
@@ -39,7 +45,8 @@ class ParallelMixer(Mixer):
         return [WeightSpec(name, (self.hidden_size,), "norm") for name in self.norm_names]
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
-        self.w_left, self.w_right = (tensors[name].to(torch.float32).contiguous() for name in self.norm_names)
+        if self.scales is None:
+            self.w_left, self.w_right = (tensors[name].to(torch.float32).contiguous() for name in self.norm_names)
         self.rt = rt
 
     def cache_needs(self) -> CacheNeeds:
@@ -69,5 +76,8 @@ class ParallelMixer(Mixer):
         b, b_bias = self._pieces(self.right.forward(h, ctx, rv, writes_cache))
         out = ctx.ws.get("parallel.out", (h.shape[0], self.hidden_size), torch.float32)
         with ctx.timed("parallel_join"):
-            ops.pair_norm_mean(a, a_bias, b, b_bias, self.w_left, self.w_right, self.eps, out)
+            if self.scales is None:
+                ops.pair_norm_mean(a, a_bias, b, b_bias, self.w_left, self.w_right, self.eps, out)
+            else:
+                ops.scaled_branches(a, a_bias, None, self.scales[0], b, b_bias, None, self.scales[1], out)
         return out

@@ -32,8 +32,9 @@ class Architecture:
     options: Dict[str, Any] = field(default_factory=dict)   # the options ``build`` understands, with their defaults
     split_fused: Optional[Callable] = None           # (config, name, tensor) -> [(name, tensor)] or None
     ignore_tensor: Optional[Callable] = None         # (config, name) -> bool
-    # (config, names of the checkpoint's tensors) -> options that the checkpoint decides (e.g. tied embeddings
-    # when the head's tensor is absent); explicit options win over them
+    # (config, the checkpoint's tensors: a set of names, or name -> shape) -> options that the checkpoint decides
+    # (e.g. tied embeddings when the head's tensor is absent, a size that only a tensor's shape gives); explicit
+    # options win over them
     checkpoint_options: Optional[Callable] = None
     # (config, flags) -> (config, options): the front end's flags (the reference's command-line and ``LLM``
     # argument names) as this architecture understands them; flags it does not know must be refused
@@ -48,7 +49,8 @@ class Architecture:
         """The model for ``config``: defaults, then what the checkpoint decides, then the given options."""
         opts = dict(self.options)
         if checkpoint_names is not None and self.checkpoint_options is not None:
-            opts.update(self.checkpoint_options(config, set(checkpoint_names)))
+            known = dict(checkpoint_names) if isinstance(checkpoint_names, Mapping) else set(checkpoint_names)
+            opts.update(self.checkpoint_options(config, known))
         for k, v in (options or {}).items():
             if k not in self.options:
                 raise ValueError(f"architecture '{self.name}' has no option '{k}' (it has: {sorted(self.options) or 'none'})")

@@ -58,12 +58,14 @@ def stored_dtype(t: torch.dtype) -> torch.dtype:
     raise WeightError(f"checkpoint tensor of unsupported dtype {t}")
 
 
-def checkpoint_names(model_dir: str) -> List[str]:
+def checkpoint_names(model_dir: str) -> Dict[str, Tuple[int, ...]]:
+    """The checkpoint's tensors without their data: name -> shape (iterating gives the names)."""
     from safetensors import safe_open
-    names: List[str] = []
+    names: Dict[str, Tuple[int, ...]] = {}
     for path in checkpoint_files(model_dir):
         with safe_open(path, framework="pt", device="cpu") as f:
-            names.extend(f.keys())
+            for name in f.keys():
+                names[name] = tuple(f.get_slice(name).get_shape())
     return names
 
 
