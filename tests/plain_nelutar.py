@@ -195,11 +195,13 @@ def expert(h, W, p, limit):
     return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ W[p + "down"].T
 
 
-def route(h, W, p, r):
-    """(chosen experts [T, top], weights [T, top])."""
+def route(h, W, p, r, margins=None):
+    """(chosen experts [T, top], weights [T, top]).  ``margins`` (a list) receives, per token, how clear the choice
+    was: the smallest gap between what was taken and what was left, among the groups and among the experts."""
     E, top = int(r["experts"]), int(r["top"])
     s = torch.sigmoid(h @ W[p + "router"].T)
     c = s + W[p + "correction"] if (p + "correction") in W else s.clone()
+    clear = torch.full((h.shape[0],), math.inf, dtype=F64)
     groups = r.get("groups")
     if groups:
         count, keep = int(groups["count"]), int(groups["keep"])
@@ -207,16 +209,25 @@ def route(h, W, p, r):
         score = per.topk(min(2, E // count), -1).values.sum(-1)
         kept = torch.zeros_like(score, dtype=torch.bool)
         kept.scatter_(1, score.topk(keep, -1).indices, True)
+        if keep < count:
+            ranked = score.sort(-1, descending=True).values
+            clear = torch.minimum(clear, ranked[:, keep - 1] - ranked[:, keep])
         c = per.masked_fill(~kept[:, :, None], -math.inf).reshape(-1, E)
     idx = c.topk(top, -1).indices
+    if top < E:
+        ranked = c.sort(-1, descending=True).values
+        gap = ranked[:, top - 1] - ranked[:, top]
+        clear = torch.minimum(clear, torch.where(torch.isfinite(gap), gap, torch.full_like(gap, math.inf)))
+    if margins is not None:
+        margins.append(clear)
     w = s.gather(1, idx)
     return idx, w / (w.sum(-1, keepdim=True) + 1e-20) * float(r.get("scale", 1.0))
 
 
-def feed_forward(h, W, p, mlp):
+def feed_forward(h, W, p, mlp, margins=None):
     if mlp["kind"] == "dense":
         return (silu(h @ W[p + "gate"].T) * (h @ W[p + "up"].T)) @ W[p + "down"].T
-    idx, w = route(h, W, p, mlp["router"])
+    idx, w = route(h, W, p, mlp["router"], margins)
     out = torch.zeros(h.shape[0], W[p + "e0.down"].shape[0], dtype=F64)
     for t in range(h.shape[0]):
         for e, a in zip(idx[t].tolist(), w[t]):
@@ -229,8 +240,9 @@ def feed_forward(h, W, p, mlp):
 MIXERS = {"parallel": parallel_mixer, "retention": retention, "parallel_2": parallel_2_mixer}
 
 
-def forward(raw, tensors, tokens, return_layers=False):
-    """Logits [T, vocab] of one sequence (and the residual after every layer run)."""
+def forward(raw, tensors, tokens, return_layers=False, margins=None):
+    """Logits [T, vocab] of one sequence (and the residual after every layer run).  ``margins`` (a list) receives one
+    tensor [T] for every routed layer run: how clear each token's choice of experts was (route)."""
     W = {k: v.to(F64) for k, v in tensors.items()}
     eps = float(raw["norm"]["eps"])
     x = embed(tokens, W, (raw.get("embedding") or {}).get("bigram"))
@@ -240,7 +252,7 @@ def forward(raw, tensors, tokens, return_layers=False):
         h = rms(x, eps) * W[p + "norm1"]
         y = W[p + "ls1"] * MIXERS[layer["type"]](h, W, p + "mix.", layer["mixer"], eps)
         if layer.get("mlp") is not None:
-            y = y + W[p + "ls2"] * feed_forward(h, W, p + "mlp.", layer["mlp"])
+            y = y + W[p + "ls2"] * feed_forward(h, W, p + "mlp.", layer["mlp"], margins)
         x = x + y
         after.append(x)
     logits = (rms(x, eps) * W["final.norm"]) @ W["head"].T
