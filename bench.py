@@ -172,7 +172,7 @@ def main():
     ap.add_argument("--perf", action="store_true",
                     help="after the timed runs, a few eager steps with the engine's timers on: average ms by kernel "
                          "class (products / attention / selection / norms / head) on stderr and under 'timers'")
-    ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k", "duvulix", "gumodra", "sagedra"],
+    ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k", "duvulix", "gumodra", "sagedra", "nelutar"],
                     help="headline: the 8B shape at batch 8, context 4,096 (the default line); "
                          "small_batch64: the 0.5B shape, 64 unequal prompts through the generation loop; sparse32k: "
                          "the 8B shape with InfLLM-v2 at 32k context; duvulix: four Duvulix layers of a real model's "
@@ -181,7 +181,9 @@ def main():
                          "four Gumodra layers of a real model's sizes (windowed attention with a sink, mLSTM, dense and "
                          "routed feed-forwards) beside the four Duvulix layers; sagedra: four Sagedra layers of a real model's sizes "
                          "(differential attention, windowed attention beside a gated delta rule, four residual streams) "
-                         "beside the four Gumodra layers")
+                         "beside the four Gumodra layers; nelutar: four Nelutar layers of a real model's sizes (capped windowed "
+                         "attention beside linear attention, windowed attention beside a delta rule with a decay a key "
+                         "channel, retention, routed experts, a layer that runs twice) beside the four Sagedra layers")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path exists)")
@@ -537,6 +539,86 @@ def sagedra_step_bytes(raw, esize, batch, context):
     return weights * esize + batch * per_seq, weights
 
 
+def config_nelutar():
+    """Four layers of sizes that resemble a real model's: width 4,096, a bigram table of 100,003 buckets; a pair of
+    capped windowed attention (32 heads on 8 kv heads of 128, 64 rotated features, 4 convolution taps, a window of
+    2,048) beside linear attention of 32 heads of 128 by 128 with fixed decays, and a SiLU-gated feed-forward of
+    11,008; a pair of windowed attention beside a delta rule with a decay a key channel (32 heads on 16 key heads,
+    128 by 128, 4 taps, decay and gate through products of rank 512) with 64 experts of 1,408 in 8 groups (4 kept),
+    6 a token, and a shared expert of 2,816; retention of 32 heads of 128 by 128 with the same experts; and the
+    second layer's weights once more."""
+    left = {"heads": 32, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 2048}}
+    decays = [1.0 - 2.0 ** (-5.0 - 3.0 * h / 31.0) for h in range(32)]
+    dense = {"kind": "dense", "ff": 11008}
+    moe = {"kind": "moe", "expert": {"ff": 1408, "limit": 7.0},
+           "router": {"experts": 64, "top": 6, "scale": 2.5, "groups": {"count": 8, "keep": 4}},
+           "shared": {"ff": 2816, "limit": 7.0}}
+    pair = {"left": dict(left, rot={"base": 500000.0, "dims": 128}),
+            "right": {"heads": 32, "kv_heads": 16, "dim": 128, "vdim": 128, "conv": 4}}
+    return {
+        "architecture": "Nelutar", "vocab": 73448, "width": 4096, "norm": {"eps": 1e-6},
+        "embedding": {"bigram": {"buckets": 100003, "mul_prev": 36313, "mul_cur": 27191}},
+        "layers": [
+            {"type": "parallel_2", "mixer": {
+                "left": dict(left, rot={"base": 10000.0, "dims": 64}, conv=4, softcap=30.0),
+                "right": {"heads": 32, "dim": 128, "vdim": 128, "decay": decays}, "left_scale": 0.6, "right_scale": 0.5},
+             "mlp": dense},
+            {"type": "parallel", "mixer": pair, "mlp": moe},
+            {"type": "retention", "mixer": {"heads": 32, "dim": 128, "vdim": 128, "decay": decays,
+                                            "rot": {"base": 1000000.0, "dims": 128}}, "mlp": moe},
+            {"type": "parallel", "mixer": pair, "mlp": moe, "weights_of": 1},
+        ],
+    }
+
+
+def nelutar_step_bytes(raw, esize, batch, context, prefill=False):
+    """Bytes a decode step must move: every matrix that the step reads once (a layer that borrows weights reads them
+    again; of a mixture: the router, the shared expert, and an expert for every (token, choice) pair, at most all of
+    them), and per sequence what its mixers read: keys and values of the window, the recurrent states read and
+    written, the convolutions' last inputs.  With ``prefill``: the matrix elements a prompt token is multiplied with
+    (of a mixture: the chosen experts only)."""
+    W = raw["width"]
+    weights = raw["vocab"] * W
+    per_seq = W * esize                                              # the bigram table's row
+    for layer in raw["layers"]:
+        m = layer["mixer"]
+
+        def attention(a):
+            nonlocal weights, per_seq
+            weights += (2 * a["heads"] * a["dim"] + a["kv_heads"] * (a["dim"] + a["vdim"])) * W
+            seen = context if not a.get("mask") else min(context, a["mask"]["size"])
+            per_seq += seen * a["kv_heads"] * (a["dim"] + a["vdim"]) * esize
+            if a.get("conv"):
+                per_seq += 2 * 4 * (a["conv"] - 1) * (a["heads"] * a["dim"] + a["kv_heads"] * (a["dim"] + a["vdim"]))
+
+        def decay_attention(d):
+            nonlocal weights, per_seq
+            weights += (2 * d["heads"] * d["dim"] + 3 * d["heads"] * d["vdim"]) * W
+            per_seq += 2 * 4 * d["heads"] * d["dim"] * d["vdim"]
+
+        if layer["type"] == "retention":
+            decay_attention(m)
+        else:
+            attention(m["left"])
+            if layer["type"] == "parallel_2":
+                decay_attention(m["right"])
+            else:
+                d = m["right"]
+                hk, hv = d["kv_heads"] * d["dim"], d["heads"] * d["vdim"]
+                ra, rg = d["heads"] * d["dim"] // 8, hv // 8
+                weights += (2 * hk + 2 * hv + d["heads"] + ra + rg) * W + ra * d["heads"] * d["dim"] + rg * hv
+                per_seq += 2 * 4 * (d["heads"] * d["dim"] * d["vdim"] + (d["conv"] - 1) * (2 * hk + hv))
+        mlp = layer.get("mlp")
+        if mlp and mlp["kind"] == "dense":
+            weights += 3 * mlp["ff"] * W
+        elif mlp:
+            r = mlp["router"]
+            weights += r["experts"] * W + (3 * mlp["shared"]["ff"] * W if mlp.get("shared") else 0)
+            pairs = r["top"] if prefill else min(max(batch, 1) * r["top"], r["experts"])
+            weights += pairs * 3 * mlp["expert"]["ff"] * W
+    return weights * esize + batch * per_seq, weights
+
+
 def duvulix_scenario(args, dev):
     """Decode and prefill of the Duvulix layer shapes beside the MiniCPM4-8B layer shape (equal width, equal
     number of layers, random weights): one JSON line with both models' figures and their timers by kernel class."""
@@ -553,6 +635,13 @@ def sagedra_scenario(args, dev):
     """The same for the Sagedra layer shapes beside the Gumodra layer shapes (the package's closest design: windowed
     attention beside a matrix-state recurrence; equal width, vocabulary and number of layers)."""
     layer_shapes_scenario(args, dev, "sagedra", "Sagedra", config_sagedra(), ("gumodra", config_gumodra()))
+
+
+def nelutar_scenario(args, dev):
+    """The same for the Nelutar layer shapes beside the Sagedra layer shapes (the package's closest design: windowed
+    attention beside a gated delta rule, layers whose weights run more than once; equal width, vocabulary and number
+    of layers)."""
+    layer_shapes_scenario(args, dev, "nelutar", "Nelutar", config_nelutar(), ("sagedra", config_sagedra()))
 
 
 def layer_shapes_scenario(args, dev, first, title, first_raw, other):
@@ -586,7 +675,8 @@ def layer_shapes_scenario(args, dev, first, title, first_raw, other):
             for grp in eng.cache.groups:
                 for st in list(grp.storage.values()) + list(grp.state.values()):
                     for t in st.values():
-                        t.normal_(0.0, 0.5)
+                        if t.is_floating_point():
+                            t.normal_(0.0, 0.5)
             return slots
 
         def decode(batch, steps, warmup):
@@ -629,6 +719,10 @@ def layer_shapes_scenario(args, dev, first, title, first_raw, other):
         elif name == "sagedra":
             step_bytes = lambda b: sagedra_step_bytes(raw, esize, b, args.context)[0]
             params = sagedra_step_bytes(raw, esize, 0, 0)[1]
+        elif name == "nelutar":
+            step_bytes = lambda b: nelutar_step_bytes(raw, esize, b, args.context)[0]
+            params = nelutar_step_bytes(raw, esize, args.batch, 0)[1]
+            prefill_params = nelutar_step_bytes(raw, esize, 1, 0, prefill=True)[1]
         else:
             step_bytes = lambda b: weight_bytes_per_step(cfg, esize) + b * args.context * kv_bytes_per_token(cfg, esize)
             params = weight_bytes_per_step(cfg, esize) // esize
@@ -687,6 +781,9 @@ def other_scenarios(args, dev):
         return
     if args.scenario == "sagedra":
         sagedra_scenario(args, dev)
+        return
+    if args.scenario == "nelutar":
+        nelutar_scenario(args, dev)
         return
     import torch
     from cpmcu_amd import Engine, EngineOptions, StepEntry

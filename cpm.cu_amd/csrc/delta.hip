@@ -110,7 +110,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
             const int e = threadIdx.x + k * 256;
             qs[e / NS][e % NS] = rq[k];
             ks[e / NS][e % NS] = rk[k];
-            if (RULE == RULE_CHANNEL) gcs[e / NS][e % NS] = expf(-A * delta_softplus(rg[k]));
+            // (rows of the tile that this step does not bring are never walked: no exponentials for them)
+            if (RULE == RULE_CHANNEL && e / NS < tn) gcs[e / NS][e % NS] = expf(-A * delta_softplus(rg[k]));
         }
 #pragma unroll
         for (int k = 0; k < VV; ++k) {

@@ -26,7 +26,7 @@ __device__ inline float silu_f(float z) { return z / (1.0f + expf(-z)); }
 // gate_after == 0; with gate_after the statistics are those of x alone and the result is multiplied by sigmoid(z)
 // (gate_after == 1) or by silu(z) (gate_after == 2)
 template <typename XT, typename ZT, typename OT>
-__global__ __launch_bounds__(256) void rms_norm_groups_kernel(const XT* __restrict__ x, long ldx,
+__global__ __launch_bounds__(1024) void rms_norm_groups_kernel(const XT* __restrict__ x, long ldx,
                                                               const ZT* __restrict__ z, long ldz,
                                                               const float* __restrict__ weight, OT* __restrict__ out,
                                                               long ldo, int W, float eps, int gate_after,
@@ -67,7 +67,9 @@ extern "C" const char* cpmcu_rms_norm_groups(const void* x, long ldx, int x_dtyp
     CPMCU_REQUIRE(ldx >= (long)groups * W && ldo >= (long)groups * W && (!z || ldz >= (long)groups * W),
                   "rms_norm_groups: leading dimensions too small for %d groups of %d", groups, W);
     dim3 grid(n, groups);
-    const int block = W >= 256 ? 256 : 64;
+    // a group as wide as a model (one norm over all heads) on few rows is a handful of workgroups, each a chain of
+    // dependent passes over its row: 1,024 threads shorten the chain
+    const int block = (W >= 2048 && (long)n * groups < 1024) ? 1024 : (W >= 256 ? 256 : 64);
 #define LAUNCH(XT, ZT, OT)                                                                                     \
     rms_norm_groups_kernel<XT, ZT, OT><<<grid, block, 0, stream>>>((const XT*)x, ldx, (const ZT*)z, ldz, weight, \
                                                                    (OT*)out, ldo, W, eps, gate_after, divisor)
