@@ -43,20 +43,36 @@ def models(tmp_path_factory):
     return out
 
 
+def deviation(got, ref):
+    """A position's deviation as the bfloat16 checks measure it: root mean square of the logits' difference (its mean
+    taken off) against the spread of the request's logits."""
+    d = got - ref
+    return (d - d.mean(1, keepdim=True)).pow(2).mean(1).sqrt() / ref.std()
+
+
 class Reference:
     """The plain implementation's logits of a request, and which of its positions chose their experts by a margin
-    that bfloat16's rounding of the router's input can overturn."""
+    that bfloat16's rounding of the router's input can overturn.  With ``conditioning`` also how far every position's
+    logits move, in float64, when every matrix is disturbed by relative noise of bfloat16's size (2^-9): what a model
+    with random weights and extreme constants (a head that keeps nothing of the past in front of a norm that divides
+    by the head's own size, keys of 8 features) does to rounding at some positions whoever computes it."""
 
-    def __init__(self, cfg, w, tokens):
+    def __init__(self, cfg, w, tokens, conditioning=False):
         margins = []
         self.logits = plain.forward(cfg, w, tokens, margins=margins).float()
         self.close = torch.zeros(len(tokens), dtype=torch.bool)
         for m in margins:
             self.close |= m < CLOSE_CALL
+        self.moved = torch.zeros(len(tokens))
+        if conditioning:
+            g = torch.Generator().manual_seed(1)
+            noisy = {k: v.double() * (1 + torch.randn(v.shape, generator=g, dtype=torch.float64) * 2.0 ** -9) if v.dim() == 2 else v
+                     for k, v in w.items()}
+            self.moved = deviation(plain.forward(cfg, noisy, tokens).float(), self.logits)
 
     def rows(self, rows):
         out = Reference.__new__(Reference)
-        out.logits, out.close = self.logits[rows], self.close[rows]
+        out.logits, out.close, out.moved = self.logits[rows], self.close[rows], self.moved[rows]
         return out
 
 
@@ -81,23 +97,24 @@ def check(got, refs, dtype, what):
     position's logits (mean taken off) against the logits' spread: 0.08 at most and 0.04 in the median.  A position
     whose choice of experts was a close call in the plain implementation (Reference.close) may have gone to other
     experts in bfloat16 and is held to 0.5 only, and so is at most one position in fifty (or one) behind such a
-    position, which reads its keys, values and state; the float32 engine is held to every position."""
+    position, which reads its keys, values and state; where the reference knows how far noise of bfloat16's size
+    moves a position in float64 (Reference.moved), the bound grows by six times that; the float32 engine is held to
+    every position."""
     for r, ref in refs.items():
         if isinstance(ref, Reference):
-            ref, close = ref.logits, ref.close
+            ref, close, moved = ref.logits, ref.close, ref.moved
         else:
-            close = torch.zeros(ref.shape[0], dtype=torch.bool)
+            close, moved = torch.zeros(ref.shape[0], dtype=torch.bool), torch.zeros(ref.shape[0])
         if dtype == "float32":
             err = (got[r] - ref).abs().max(dim=1).values
             bad = (err > 2e-4 * max(1.0, float(ref.abs().max()))).nonzero().flatten()
             assert bad.numel() == 0, (f"{what}: request {r}: first wrong position {int(bad[0])} of {ref.shape[0]} "
                                       f"(error {float(err[bad[0]]):.3g})")
             continue
-        d = got[r] - ref
-        err = (d - d.mean(1, keepdim=True)).pow(2).mean(1).sqrt() / ref.std()
-        over = ((err > 0.08) & ~close).nonzero().flatten()
+        err = deviation(got[r], ref)
+        over = ((err > 0.08 + 6.0 * moved) & ~close).nonzero().flatten()
         allowed = max(1, ref.shape[0] // 50) if (bool(close.any()) and over.numel() and int(over[0]) > int(close.nonzero()[0])) else 0
-        assert over.numel() <= allowed and float(err.max()) <= 0.5 and float(err.median()) <= 0.04, \
+        assert over.numel() <= allowed and float((err - 6.0 * moved).max()) <= 0.5 and float(err.median()) <= 0.04 + float(moved.median()), \
             (f"{what}: request {r}: {over.numel()} of {ref.shape[0]} positions over 0.08 whose choice of experts was "
              f"clear (first {int(over[0]) if over.numel() else -1}, worst {float(err.max()):.3g}, median "
              f"{float(err.median()):.3g}; close calls at {close.nonzero().flatten().tolist()[:12]})")
