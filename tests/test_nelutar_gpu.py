@@ -96,10 +96,10 @@ def check(got, refs, dtype, what):
     """float32 (the sharp comparison): rounding of float sums, at every position.  bfloat16: the deviation of a
     position's logits (mean taken off) against the logits' spread: 0.08 at most and 0.04 in the median.  A position
     whose choice of experts was a close call in the plain implementation (Reference.close) may have gone to other
-    experts in bfloat16 and is held to 0.5 only, and so is at most one position in fifty (or one) behind such a
-    position, which reads its keys, values and state; where the reference knows how far noise of bfloat16's size
-    moves a position in float64 (Reference.moved), the bound grows by six times that; the float32 engine is held to
-    every position."""
+    experts in bfloat16 and is not held to a bound, and at most one position in fifty (or one) behind such a
+    position, which reads its keys, values and state, is held to 0.5 only; where the reference knows how far noise of
+    bfloat16's size moves a position in float64 (Reference.moved), the bound grows by six times that; the float32
+    engine is held to every position."""
     for r, ref in refs.items():
         if isinstance(ref, Reference):
             ref, close, moved = ref.logits, ref.close, ref.moved
@@ -114,7 +114,8 @@ def check(got, refs, dtype, what):
         err = deviation(got[r], ref)
         over = ((err > 0.08 + 6.0 * moved) & ~close).nonzero().flatten()
         allowed = max(1, ref.shape[0] // 50) if (bool(close.any()) and over.numel() and int(over[0]) > int(close.nonzero()[0])) else 0
-        assert over.numel() <= allowed and float((err - 6.0 * moved).max()) <= 0.5 and float(err.median()) <= 0.04 + float(moved.median()), \
+        clear = (err - 6.0 * moved)[~close]
+        assert over.numel() <= allowed and (clear.numel() == 0 or float(clear.max()) <= 0.5) and float(err.median()) <= 0.04 + float(moved.median()), \
             (f"{what}: request {r}: {over.numel()} of {ref.shape[0]} positions over 0.08 whose choice of experts was "
              f"clear (first {int(over[0]) if over.numel() else -1}, worst {float(err.max()):.3g}, median "
              f"{float(err.median()):.3g}; close calls at {close.nonzero().flatten().tolist()[:12]})")
@@ -384,3 +385,24 @@ def test_a_long_sequence(models, name, dtype):
     eng.release(s)
     rows = want + list(range(1260, 1300))
     check({"long": torch.cat(got)}, {"long": ref.rows(rows)}, dtype, "a long sequence")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_of_a_real_models_kind(dtype, tmp_path):
+    """Width 1,024 and heads of 128: a prompt of 330 tokens (the library's products, attention and experts on the
+    matrix cores, a window of 256 that has passed the first tokens), then 24 tokens one by one through captured
+    graphs (strip and skinny products), and a batch of three unequal requests."""
+    from cpmcu_amd import Engine, EngineOptions
+    raw = tn.medium_m()
+    d = str(tmp_path / "m")
+    tn.write_model(raw, d, 301, std=0.03)
+    cfg, w = tiny.read_model(d)
+    reqs = {"a": tiny.random_tokens(354, raw["vocab"], 3100), "b": tiny.random_tokens(70, raw["vocab"], 3101),
+            "c": tiny.random_tokens(9, raw["vocab"], 3102)}
+    refs = {r: Reference(cfg, w, t, conditioning=(dtype == "bfloat16")) for r, t in reqs.items()}
+    eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=1024, max_slots=3, max_seq_len=512, hip_graph=True))
+    check(schedules.tail(eng, {"a": reqs["a"]}, 24), {"a": refs["a"]}, dtype, "prompt of 330, then 24 tokens")
+    got = schedules.batched(eng, reqs, {"a": 300, "b": 66, "c": 2}, [("c", "a", "b")])
+    check(got, refs, dtype, "batch of three")
+    eng.cache.check()
+    assert not eng.cache.live

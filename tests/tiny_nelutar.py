@@ -114,6 +114,32 @@ def tiny_r():
     }
 
 
+def medium_m():
+    """Sizes of a real model's kind, so that the kernels for aligned sizes run (matrix-core attention with heads of
+    128, strip and skinny products, the library's product, experts on the matrix cores, 16 state values a lane): width
+    1,024, heads of 128 by 128, windows of 256, 8 experts of 512 with a shared one, ranks of 64 (by the writer's
+    rule)."""
+    left = {"heads": 8, "kv_heads": 2, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 256}}
+    moe = {"kind": "moe", "expert": {"ff": 512, "limit": 4.0},
+           "router": {"experts": 8, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}, "shared": {"ff": 512, "limit": 4.0}}
+    decays = [0.9, 0.97, 0.99, 0.999]
+    return {
+        "architecture": "Nelutar", "vocab": 1000, "width": 1024, "norm": {"eps": 1e-6},
+        "embedding": {"bigram": {"buckets": 4099, "mul_prev": 1009, "mul_cur": 757}},
+        "layers": [
+            {"type": "parallel_2", "mixer": {
+                "left": dict(left, rot={"base": 10000.0, "dims": 64}, conv=4, softcap=30.0),
+                "right": {"heads": 4, "dim": 128, "vdim": 128, "decay": decays}, "left_scale": 0.6, "right_scale": 0.5},
+             "mlp": {"kind": "dense", "ff": 2048}},
+            {"type": "parallel", "mixer": {"left": dict(left, rot={"base": 500000.0, "dims": 128}),
+                                           "right": {"heads": 4, "kv_heads": 2, "dim": 128, "vdim": 128, "conv": 4}},
+             "mlp": moe},
+            {"type": "retention", "mixer": {"heads": 4, "dim": 128, "vdim": 128, "decay": decays,
+                                            "rot": {"base": 1000000.0, "dims": 128}}, "mlp": moe},
+        ],
+    }
+
+
 def write_model(raw, out_dir, seed, std=0.08, norm_std=0.1):
     """A model folder with random weights through the package's own writer; config.json is the raw dictionary."""
     import cpmcu_amd
