@@ -290,15 +290,23 @@ class NelutarConfig(ModelConfig):
                     "config.json embedding bigram: buckets must be positive, the multipliers not negative")
         layers = raw.get("layers")
         require(isinstance(layers, list) and len(layers) > 0, "config.json: 'layers' must be a non-empty list")
-        parsed = tuple(LayerConfig.from_dict(l, i) for i, l in enumerate(layers))
+        # a layer that uses another's weights equals it in everything else: what its entry leaves out is the other's
+        filled = []
+        for i, l in enumerate(layers):
+            j = l.get("weights_of") if isinstance(l, dict) else None
+            if isinstance(j, int) and not isinstance(j, bool) and 0 <= j < len(layers) and j != i and isinstance(layers[j], dict):
+                l = {**{k: v for k, v in layers[j].items() if k != "weights_of"}, **l}
+            filled.append(l)
+        parsed = tuple(LayerConfig.from_dict(l, i) for i, l in enumerate(filled))
         for i, l in enumerate(parsed):
             if l.weights_of is None:
                 continue
             j = l.weights_of
             require(0 <= j < len(parsed) and j != i and parsed[j].weights_of is None,
                     f"config.json layers[{i}]: weights_of ({j}) must name another layer that has weights of its own")
-            require((l.type, l.mixer, l.mlp) == (parsed[j].type, parsed[j].mixer, parsed[j].mlp),
-                    f"config.json layers[{i}]: a layer that uses layer {j}'s weights must equal it in type, mixer and mlp")
+            require(l.type == parsed[j].type and (l.mlp is None) == (parsed[j].mlp is None) and
+                    (l.mlp is None or l.mlp.kind == parsed[j].mlp.kind),
+                    f"config.json layers[{i}]: a layer that uses layer {j}'s weights must equal it in type and kind of mlp")
         return cls(ARCHITECTURE, vocab, width, eps, bigram, parsed)
 
     def to_dict(self) -> Dict[str, Any]:
@@ -311,6 +319,16 @@ class NelutarConfig(ModelConfig):
     def layer_weights(self) -> Tuple[int, ...]:
         """For every layer, the layer whose tensors it uses (itself, unless it says otherwise)."""
         return tuple(i if l.weights_of is None else l.weights_of for i, l in enumerate(self.layers))
+
+    def shares_block(self, i: int) -> bool:
+        """Whether layer i is its weights' owner run once more: it borrows, and equals the owner in every size and
+        constant (what a borrowing layer is meant to be; one that differs, in a window or a decay, say, is built as a
+        layer of its own that reads the owner's tensors)."""
+        l = self.layers[i]
+        if l.weights_of is None:
+            return False
+        o = self.layers[l.weights_of]
+        return (l.type, l.mixer, l.mlp) == (o.type, o.mixer, o.mlp)
 
     @property
     def vocabulary_size(self) -> int:

@@ -58,10 +58,12 @@ def _channel_delta(cfg: NelutarConfig, m, p: str, ranks):
 
 
 def _mixer(cfg: NelutarConfig, i: int, options):
-    layer, p = cfg.layers[i], f"l{i}.mix."
+    """The mixer of layer i, reading the tensors of the layer whose weights it uses."""
+    layer, w = cfg.layers[i], cfg.layer_weights()[i]
+    p = f"l{w}.mix."
     m = layer.mixer
     if layer.type == "parallel":
-        ranks = options.get(f"l{i}.ranks", (max(m.right.heads * m.right.dim // 8, 1), max(m.right.heads * m.right.vdim // 8, 1)))
+        ranks = options.get(f"l{w}.ranks", (max(m.right.heads * m.right.dim // 8, 1), max(m.right.heads * m.right.vdim // 8, 1)))
         return MIXERS.build("parallel", left=_attention(cfg, m.left, p + "left.", normed=False),
                             right=_channel_delta(cfg, m.right, p + "right.", ranks), left_norm_name=p + "left.out",
                             right_norm_name=p + "right.out", hidden_size=cfg.width, eps=cfg.eps)
@@ -81,7 +83,7 @@ def _mixer(cfg: NelutarConfig, i: int, options):
 
 
 def _feed_forward(cfg: NelutarConfig, i: int):
-    ff, p = cfg.layers[i].mlp, f"l{i}.mlp."
+    ff, p = cfg.layers[i].mlp, f"l{cfg.layer_weights()[i]}.mlp."
     if ff is None:
         return None
     if ff.kind == "dense":
@@ -103,14 +105,16 @@ def build(cfg: NelutarConfig, ranks=None) -> DecoderModel:
     norm = lambda name: NORMS.build("rms_norm", name=name, hidden_size=cfg.width, eps=cfg.eps)
     owner = cfg.layer_weights()
     blocks, index = [], {}
-    for i in sorted(set(owner)):
-        p = f"l{i}."
+    for i in range(len(cfg.layers)):
+        if cfg.shares_block(i):
+            continue                    # the owner's block runs once more
+        p = f"l{owner[i]}."
         ff = _feed_forward(cfg, i)
         index[i] = len(blocks)
         blocks.append(BLOCKS.build("parallel_scaled", norm=norm(p + "norm1"), mixer=_mixer(cfg, i, options), feed_forward=ff,
                                    hidden_size=cfg.width, scale_names=[p + "ls1"] + ([p + "ls2"] if ff is not None else [])))
     # every layer of the configuration is a run with a cache entry of its own, whoever's weights it uses
-    schedule = [Run(index[j], entry, True) for entry, j in enumerate(owner)]
+    schedule = [Run(index[owner[i]] if cfg.shares_block(i) else index[i], entry, True) for entry, i in enumerate(range(len(cfg.layers)))]
     bigram = ("bigram",) + tuple(cfg.bigram) if cfg.bigram is not None else None
     embedding = TokenEmbedding("embed", cfg.vocab, cfg.width, 1.0, bigram=bigram)
     head = LMHead("head", cfg.vocab, cfg.width, 1.0)

@@ -66,6 +66,7 @@ def test_defaults_of_absent_keys():
     (lambda r: r["layers"][3].update(weights_of=3), "weights_of"),
     (lambda r: r["layers"][3].update(weights_of=4), "weights_of"),
     (lambda r: r["layers"][3].update(weights_of=1), "equal"),
+    (lambda r: r["layers"][3].update(mlp=None), "equal"),
     (lambda r: r["embedding"]["bigram"].update(buckets=0), "buckets"),
     (lambda r: r.pop("norm"), "norm"),
 ])
@@ -75,6 +76,25 @@ def test_refusals(change, word):
     change(raw)
     with pytest.raises(ConfigError, match=word):
         _cfg(raw)
+
+
+def test_a_borrowing_layer_may_leave_out_what_it_shares():
+    raw = tn.tiny_p()
+    full = _cfg(raw)[1]
+    raw["layers"][3] = {"weights_of": 0}
+    raw["layers"][4] = {"type": "parallel_2", "weights_of": 2, "mixer": raw["layers"][4]["mixer"]}
+    assert _cfg(raw)[1] == full
+
+
+def test_a_borrowing_layer_that_differs_is_a_layer_of_its_own_on_the_same_tensors():
+    raw = tn.tiny_p()
+    raw["layers"][3]["mixer"]["left"]["mask"]["size"] = 9
+    arch, cfg = _cfg(raw)
+    model = arch.build_model(cfg)
+    assert len(model.layers) == 4 and [r.layer for r in model.schedule] == [0, 1, 2, 3, 2]
+    assert {s.name for s in model.layers[3].all_weight_specs()} == {s.name for s in model.layers[0].all_weight_specs()}
+    needs = model.cache_needs()
+    assert needs[0].window == 20 and needs[3].window == 9
 
 
 def test_tensor_names_and_cache_needs():

@@ -255,6 +255,25 @@ def test_borrowed_weights_are_held_once(models):
     assert [r.cache for r in eng.model.schedule] == [0, 1, 2, 3, 4] and eng.model.embedding_entry == 5
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_borrowing_layer_with_constants_of_its_own(dtype, tmp_path):
+    """A layer that uses another's tensors but differs from it (a window of 9 instead of 20, other decays): it is
+    built as a layer of its own on the owner's tensors."""
+    from cpmcu_amd import Engine, EngineOptions
+    raw = tn.tiny_p()
+    raw["layers"][3]["mixer"]["left"]["mask"]["size"] = 9
+    raw["layers"][4]["mixer"]["right"]["decay"] = [0.5, 0.9]
+    raw["layers"][4]["mixer"]["left_scale"] = 0.2
+    d = str(tmp_path / "m")
+    tn.write_model(raw, d, 311)
+    cfg, w = tiny.read_model(d)
+    reqs = {"a": tiny.random_tokens(90, raw["vocab"], 3200), "b": tiny.random_tokens(7, raw["vocab"], 3201)}
+    refs = {r: Reference(cfg, w, t) for r, t in reqs.items()}
+    eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=512, max_slots=2, max_seq_len=256))
+    assert len(eng.model.layers) == 5
+    check(schedules.tail(eng, reqs, 30), refs, dtype, "borrowed tensors, own constants")
+
+
 def _greedy(cfg, w, prompt, n):
     toks = list(prompt)
     out = []
