@@ -551,7 +551,7 @@ def config_nelutar():
     decays = [1.0 - 2.0 ** (-5.0 - 3.0 * h / 31.0) for h in range(32)]
     dense = {"kind": "dense", "ff": 11008}
     moe = {"kind": "moe", "expert": {"ff": 1408, "limit": 7.0},
-           "router": {"experts": 64, "top": 6, "scale": 2.5, "groups": {"count": 8, "keep": 4}},
+           "router": {"experts": 64, "top": 6, "scale": 2.0, "groups": {"count": 8, "keep": 4}},
            "shared": {"ff": 2816, "limit": 7.0}}
     pair = {"left": dict(left, rot={"base": 500000.0, "dims": 128}),
             "right": {"heads": 32, "kv_heads": 16, "dim": 128, "vdim": 128, "conv": 4}}
@@ -561,11 +561,11 @@ def config_nelutar():
         "layers": [
             {"type": "parallel_2", "mixer": {
                 "left": dict(left, rot={"base": 10000.0, "dims": 64}, conv=4, softcap=30.0),
-                "right": {"heads": 32, "dim": 128, "vdim": 128, "decay": decays}, "left_scale": 0.6, "right_scale": 0.5},
+                "right": {"heads": 32, "dim": 128, "vdim": 128, "decay": decays}, "left_scale": 0.7, "right_scale": 0.4},
              "mlp": dense},
             {"type": "parallel", "mixer": pair, "mlp": moe},
             {"type": "retention", "mixer": {"heads": 32, "dim": 128, "vdim": 128, "decay": decays,
-                                            "rot": {"base": 1000000.0, "dims": 128}}, "mlp": moe},
+                                            "rot": {"base": 100000.0, "dims": 128}}, "mlp": moe},
             {"type": "parallel", "mixer": pair, "mlp": moe, "weights_of": 1},
         ],
     }

@@ -88,7 +88,7 @@ def draw(seed):
     raw = {"architecture": "Nelutar", "vocab": rng.randint(50, 300), "width": rng.choice([64, 72, 96, 128, 160]),
            "norm": {"eps": rng.choice([1e-5, 1e-6])}, "layers": []}
     if rng.random() < 0.7:
-        raw["embedding"] = {"bigram": {"buckets": rng.choice([1, 31, 509]), "mul_prev": rng.randint(0, 40), "mul_cur": rng.randint(1, 40)}}
+        raw["embedding"] = {"bigram": {"buckets": rng.choice([1, 31, 251]), "mul_prev": rng.randint(0, 40), "mul_cur": rng.randint(1, 40)}}
     ranks = {}
     for i in range(rng.randint(3, 5)):
         own = [j for j, l in enumerate(raw["layers"]) if "weights_of" not in l]

@@ -129,13 +129,13 @@ def medium_m():
         "layers": [
             {"type": "parallel_2", "mixer": {
                 "left": dict(left, rot={"base": 10000.0, "dims": 64}, conv=4, softcap=30.0),
-                "right": {"heads": 4, "dim": 128, "vdim": 128, "decay": decays}, "left_scale": 0.6, "right_scale": 0.5},
+                "right": {"heads": 4, "dim": 128, "vdim": 128, "decay": decays}, "left_scale": 0.7, "right_scale": 0.4},
              "mlp": {"kind": "dense", "ff": 2048}},
             {"type": "parallel", "mixer": {"left": dict(left, rot={"base": 500000.0, "dims": 128}),
                                            "right": {"heads": 4, "kv_heads": 2, "dim": 128, "vdim": 128, "conv": 4}},
              "mlp": moe},
             {"type": "retention", "mixer": {"heads": 4, "dim": 128, "vdim": 128, "decay": decays,
-                                            "rot": {"base": 1000000.0, "dims": 128}}, "mlp": moe},
+                                            "rot": {"base": 100000.0, "dims": 128}}, "mlp": moe},
         ],
     }
 
