@@ -265,7 +265,7 @@ def test_a_borrowing_layer_with_constants_of_its_own(dtype, tmp_path):
     raw["layers"][4]["mixer"]["right"]["decay"] = [0.5, 0.9]
     raw["layers"][4]["mixer"]["left_scale"] = 0.2
     d = str(tmp_path / "m")
-    tn.write_model(raw, d, 311)
+    tn.write_model(raw, d, 311, router_gain=5.0)
     cfg, w = tiny.read_model(d)
     reqs = {"a": tiny.random_tokens(90, raw["vocab"], 3200), "b": tiny.random_tokens(7, raw["vocab"], 3201)}
     refs = {r: Reference(cfg, w, t) for r, t in reqs.items()}

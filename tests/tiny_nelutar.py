@@ -140,8 +140,10 @@ def medium_m():
     }
 
 
-def write_model(raw, out_dir, seed, std=0.08, norm_std=0.1):
-    """A model folder with random weights through the package's own writer; config.json is the raw dictionary."""
+def write_model(raw, out_dir, seed, std=0.08, norm_std=0.1, router_gain=1.0):
+    """A model folder with random weights through the package's own writer; config.json is the raw dictionary.
+    ``router_gain`` multiplies the routers' weights: with the writer's small weights the experts' scores lie close
+    together and every other token's choice is a close call; a gain spreads them."""
     import cpmcu_amd
     from cpmcu_amd.weights import write_model_dir
     arch = cpmcu_amd.get_architecture(raw["architecture"])
@@ -149,4 +151,12 @@ def write_model(raw, out_dir, seed, std=0.08, norm_std=0.1):
     write_model_dir(cfg, out_dir, seed, std=std, norm_std=norm_std)
     with open(os.path.join(out_dir, "config.json"), "w") as f:
         json.dump(raw, f, indent=1)
+    if router_gain != 1.0:
+        from safetensors.torch import load_file, save_file
+        path = os.path.join(out_dir, "model.safetensors")
+        tensors = load_file(path)
+        for name in tensors:
+            if name.endswith(".mlp.router"):
+                tensors[name] = (tensors[name].float() * router_gain).to(tensors[name].dtype)
+        save_file(tensors, path)
     return out_dir
