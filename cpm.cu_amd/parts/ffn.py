@@ -177,7 +177,10 @@ class RoutedExpertsFFN(FeedForward):
         out = ctx.ws.get("moe.out", (n, self.hidden_size), torch.float32)
         tiles = ops.moe_tiles(n, self.top, self.experts)
         with ctx.timed("moe_experts"):
-            if n > ops.SKINNY_MAX_ROWS and ops.moe_experts_mfma_ok(h, self.expert_size, tiles):
+            # few tokens read an expert's matrices once for every token that chose it; from about one and a half
+            # (token, expert) pairs an expert on, most experts are chosen more than once and grouping pays
+            grouped = n > ops.SKINNY_MAX_ROWS or 2 * n * self.top >= 3 * self.experts
+            if grouped and ops.moe_experts_mfma_ok(h, self.expert_size, tiles):
                 # many tokens: experts are shared by many of them; pairs grouped by expert, on the matrix cores
                 y = ctx.ws.get("moe.pair_out", (n, self.top, self.hidden_size), torch.bfloat16)
                 rows = ctx.ws.get("moe.tile_rows", (tiles * ops.MOE_TILE,), torch.int32)
