@@ -34,8 +34,8 @@ from .decoder import DecoderModel, Run
 _FF_NAMES = {"gate": "gate", "up": "up", "down": "down"}
 
 
-def _rotation(m):
-    return POSITION_ENCODINGS.build("rope", head_dim=m.rot_dims, theta=m.rot_base) if m.rot_dims else None
+def _rotation(m, pairs):
+    return POSITION_ENCODINGS.build("rope", head_dim=m.rot_dims, theta=m.rot_base, pairs=pairs) if m.rot_dims else None
 
 
 def _attention(cfg: NelutarConfig, m, p: str, normed: bool):
@@ -43,9 +43,9 @@ def _attention(cfg: NelutarConfig, m, p: str, normed: bool):
     if m.conv:
         names.update({"q_conv": p + "q.conv", "k_conv": p + "k.conv", "v_conv": p + "v.conv"})
     return MIXERS.build("attention", names=names, hidden_size=cfg.width, num_heads=m.heads, num_kv_heads=m.kv_heads,
-                        key_dim=m.dim, value_dim=m.vdim, position=_rotation(m), scale=m.scale, mask_window=m.window,
-                        norm_eps=cfg.eps, unit_norm_after_rotation=normed, rotation_pairs="interleaved",
-                        score_softcap=m.softcap, conv_taps=m.conv)
+                        key_dim=m.dim, value_dim=m.vdim, position=_rotation(m, "interleaved"), scale=m.scale,
+                        mask_window=m.window, norm_eps=cfg.eps, unit_norm_after_rotation=normed, score_softcap=m.softcap,
+                        conv_taps=m.conv)
 
 
 def _channel_delta(cfg: NelutarConfig, m, p: str, ranks):
@@ -72,13 +72,13 @@ def _mixer(cfg: NelutarConfig, i: int, options):
         right = MIXERS.build("decay_linear_attention",
                              names={"q": q + "q", "k": q + "k", "v": q + "v", "gate": q + "g", "out": q + "o", "norm": q + "norm"},
                              hidden_size=cfg.width, heads=r.heads, key_dim=r.dim, value_dim=r.vdim, decay=r.decay,
-                             eps=cfg.eps, activation="silu", position=_rotation(r), rotation_pairs="interleaved",
-                             norm="all", gate_activation="sigmoid")
+                             eps=cfg.eps, activation="silu", position=_rotation(r, "interleaved"), norm="all",
+                             gate_activation="sigmoid")
         return MIXERS.build("parallel", left=_attention(cfg, m.left, p + "left.", normed=True), right=right,
                             hidden_size=cfg.width, scales=(m.left_scale, m.right_scale))
     names = {"q": p + "q", "k": p + "k", "v": p + "v", "gate": p + "g", "out": p + "o"}
     return MIXERS.build("decay_linear_attention", names=names, hidden_size=cfg.width, heads=m.heads, key_dim=m.dim,
-                        value_dim=m.vdim, decay=m.decay, eps=cfg.eps, position=_rotation(m), rotation_pairs="halves",
+                        value_dim=m.vdim, decay=m.decay, eps=cfg.eps, position=_rotation(m, "halves"),
                         key_scale=m.dim ** -0.5, norm="heads", gate_activation="silu")
 
 

@@ -41,6 +41,9 @@ class GQAAttention(Mixer):
                              f"head sizes in steps of 16 up to 256")
         self.hidden_size = hidden_size
         self.nh, self.nkv, self.hd = num_heads, num_kv_heads, head_dim
+        if position is not None and position.pairs != "halves":
+            raise ValueError(f"gqa_attention: the fused rotation pairs feature i with i + head_dim/2; an encoding of "
+                             f"'{position.pairs}' pairs belongs to the mixer kind 'attention'")
         self.position = position
         self.scale = float(scale) if scale is not None else head_dim ** -0.5
         self.qkv = Linear([(prefix + "q_proj.weight", num_heads * head_dim),
@@ -245,7 +248,8 @@ class GeneralAttention(Mixer):
                            of a sequence are fixed-size state of its cache slot.
     ``unit_norm_after_rotation``: q and k heads are divided by their root mean square (``norm_eps`` inside the
     root, no weight) after the rotation.
-    ``rotation_pairs``: 'halves' pairs feature i with i + r/2 of the r rotated features, 'interleaved' 2i with 2i + 1.
+    The rotation pairs the features that ``position.pairs`` says ('halves': i with i + r/2 of the r rotated features;
+    'interleaved': 2i with 2i + 1).
     ``score_softcap`` c: a scaled score s enters the softmax as c tanh(s / c).
     Without 'v' the values are the keys as projected (with their bias, before norm and rotation): value_dim
     must equal key_dim."""
@@ -253,8 +257,7 @@ class GeneralAttention(Mixer):
     def __init__(self, names: Mapping[str, str], hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int,
                  value_dim: int, position: Optional[PositionEncoding], scale: float, mask_chunk: Optional[int] = None,
                  mask_window: Optional[int] = None, mask_keep_first: int = 0, norm_eps: float = 0.0,
-                 unit_norm_after_rotation: bool = False, rotation_pairs: str = "halves",
-                 score_softcap: Optional[float] = None, conv_taps: int = 0):
+                 unit_norm_after_rotation: bool = False, score_softcap: Optional[float] = None, conv_taps: int = 0):
         if num_heads % num_kv_heads:
             raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         if unit_norm_after_rotation and (names.get("q_norm") or names.get("k_norm")):
@@ -269,13 +272,11 @@ class GeneralAttention(Mixer):
             raise ValueError("attention: a chunked mask or a sliding window, not both")
         if mask_keep_first < 0 or (mask_keep_first and not mask_window):
             raise ValueError("attention: kept first tokens come with a sliding window")
-        if rotation_pairs not in ("halves", "interleaved"):
-            raise ValueError(f"attention: rotation pairs '{rotation_pairs}' (halves or interleaved)")
         if score_softcap is not None and not score_softcap > 0:
             raise ValueError(f"attention: a score cap of {score_softcap}")
         if conv_taps < 0:
             raise ValueError(f"attention: {conv_taps} convolution taps")
-        self.interleaved = rotation_pairs == "interleaved"
+        self.interleaved = position is not None and position.pairs == "interleaved"
         self.softcap = float(score_softcap) if score_softcap is not None else 0.0
         self.taps = int(conv_taps)
         self.names = dict(names)

@@ -324,8 +324,12 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
+    # which features a rotation pairs: 'halves' pairs feature i with i + r/2 of the r rotated features (rotate-half),
+    # 'interleaved' pairs neighbours 2i and 2i + 1.  A mixer whose kernels know only one of them refuses the other.
+    pairs = "halves"
+
     def rotary_params(self) -> Optional[Tuple[torch.Tensor, float]]:
-        """(inv_freq float32 [head_dim/2], magnitude) if this encoding is a rotate-half rotation by
+        """(inv_freq float32 [head_dim/2], magnitude) if this encoding is a rotation of feature pairs (``pairs``) by
         position * inv_freq, which the fused kernel applies while it writes the cache; else None."""
         return None
 

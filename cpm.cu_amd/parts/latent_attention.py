@@ -86,6 +86,8 @@ class LatentAttention(Mixer):
         if self.rot and rot is None:
             raise ValueError("latent_attention: the position encoding must be a rotation (rotary_params)")
         inv_freq, mag = rot if rot is not None else (None, 1.0)
+        if self.rot and self.position.pairs != "halves":
+            raise ValueError(f"latent_attention: the rotation pairs feature i with i + rot/2, not '{self.position.pairs}'")
         if self.rot and inv_freq.shape[0] * 2 != self.rot:
             raise ValueError(f"latent_attention: the rotation covers {inv_freq.shape[0] * 2} features, the rotated "
                              f"part has {self.rot}")

@@ -7,8 +7,8 @@ One input projection gives [q: heads*dim | k: heads*dim | v: heads*vdim | gate: 
 between the projection and the recurrence, and between the recurrence and the output projection, are parameters:
 
     ``activation``       None, or 'silu' on q, k and v;
-    ``position``         a rotation of the first features of q and k heads (``rotation_pairs`` 'halves' or
-                         'interleaved'), or None;
+    ``position``         a rotation of the first features of q and k heads (of the pairs that ``position.pairs``
+                         says), or None;
     ``key_scale``        k is multiplied by it after the rotation;
     ``norm``             'heads': each head's o is divided by its own root mean square; 'all': the heads side by side are
                          divided by one root mean square; with 'norm' in ``names`` the result is multiplied by that
@@ -34,7 +34,7 @@ from .linear import Linear
 class DecayLinearAttention(Mixer):
     def __init__(self, names: Mapping[str, str], hidden_size: int, heads: int, key_dim: int, value_dim: int,
                  decay: Sequence[float], eps: float, activation: Optional[str] = None,
-                 position: Optional[PositionEncoding] = None, rotation_pairs: str = "halves", key_scale: float = 1.0,
+                 position: Optional[PositionEncoding] = None, key_scale: float = 1.0,
                  norm: str = "heads", gate_activation: str = "silu"):
         """``names``: checkpoint tensors for 'q', 'k', 'v', 'gate', 'out' and optionally 'norm'."""
         if len(decay) != heads:
@@ -45,8 +45,6 @@ class DecayLinearAttention(Mixer):
             raise ValueError(f"decay_linear_attention: a key size of {key_dim} is not supported (at most 256)")
         if activation not in (None, "silu"):
             raise ValueError(f"decay_linear_attention: activation '{activation}' (none or silu)")
-        if rotation_pairs not in ("halves", "interleaved"):
-            raise ValueError(f"decay_linear_attention: rotation pairs '{rotation_pairs}' (halves or interleaved)")
         if norm not in ("heads", "all"):
             raise ValueError(f"decay_linear_attention: norm over '{norm}' (heads or all)")
         if gate_activation not in ("silu", "sigmoid"):
@@ -55,7 +53,8 @@ class DecayLinearAttention(Mixer):
         self.hidden_size, self.heads, self.dk, self.dv = hidden_size, heads, key_dim, value_dim
         self.decay = [float(d) for d in decay]
         self.eps, self.activation, self.position = float(eps), activation, position
-        self.interleaved, self.key_scale = rotation_pairs == "interleaved", float(key_scale)
+        self.interleaved = position is not None and position.pairs == "interleaved"
+        self.key_scale = float(key_scale)
         self.norm_groups = heads if norm == "heads" else 1
         self.gate_activation = gate_activation
         n, hk, hv = self.names, heads * key_dim, heads * value_dim

@@ -1,6 +1,7 @@
 """Rotary position encoding, plain and LongRoPE.
 
-Rotate-half rotation by theta = position * inv_freq[c] (src/model/rotary.cuh:7-34).
+Rotate-half rotation by theta = position * inv_freq[c] (src/model/rotary.cuh:7-34); with ``pairs='interleaved'`` the
+plain encoding pairs neighbouring features (2c, 2c + 1) instead of (c, c + head_dim/2), with the same angles.
 The reference loads inv_freq once, computed for the engine's whole token budget
 (cpmcu/llm.py:181-191): the choice between LongRoPE's short and long factors is
 static per engine, long iff the engine holds sequences longer than
@@ -21,7 +22,10 @@ from .base import POSITION_ENCODINGS, PositionEncoding, Runtime
 
 @POSITION_ENCODINGS.register("rope")
 class RotaryEncoding(PositionEncoding):
-    def __init__(self, head_dim: int, theta: float):
+    def __init__(self, head_dim: int, theta: float, pairs: str = "halves"):
+        if pairs not in ("halves", "interleaved"):
+            raise ValueError(f"rope: pairs '{pairs}' (halves or interleaved)")
+        self.pairs = pairs
         self.head_dim = head_dim
         self.theta = float(theta)
         self.inv_freq: Optional[torch.Tensor] = None
