@@ -97,6 +97,21 @@ def test_a_borrowing_layer_that_differs_is_a_layer_of_its_own_on_the_same_tensor
     assert needs[0].window == 20 and needs[3].window == 9
 
 
+def test_the_pairing_belongs_to_the_position_encoding():
+    from cpmcu_amd.parts import MIXERS, POSITION_ENCODINGS
+    arch, cfg = _cfg(tn.tiny_p())
+    model = arch.build_model(cfg)
+    pair, retention = model.layers[0].mixer, model.layers[1].mixer
+    assert pair.left.position.pairs == "interleaved" and pair.left.interleaved
+    assert retention.position.pairs == "halves" and not retention.interleaved
+    assert POSITION_ENCODINGS.build("rope", head_dim=8, theta=10.0).pairs == "halves"
+    with pytest.raises(ValueError, match="pairs"):
+        POSITION_ENCODINGS.build("rope", head_dim=8, theta=10.0, pairs="thirds")
+    turned = POSITION_ENCODINGS.build("rope", head_dim=16, theta=100.0, pairs="interleaved")
+    with pytest.raises(ValueError, match="interleaved"):
+        MIXERS.build("gqa_attention", prefix="x.", hidden_size=64, num_heads=4, num_kv_heads=2, head_dim=16, position=turned)
+
+
 def test_tensor_names_and_cache_needs():
     arch, cfg = _cfg(tn.tiny_p())
     model = arch.build_model(cfg, {"ranks": {0: (5, 7)}})
